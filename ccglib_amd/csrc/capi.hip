@@ -1,0 +1,577 @@
+// C ABI of the library (declared in include/ccglib_amd.h): argument checking,
+// object state and stream plumbing around the kernel launchers. The host-side
+// behaviour mirrors the reference classes it replaces: src/mma/GEMM.cpp,
+// src/transpose/Transpose.cpp, src/packing/Packing.cpp,
+// src/pipeline/Pipeline.cpp.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "../../include/ccglib_amd.h"
+#include "common.h"
+
+using namespace ccglib_amd;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int fail_hip(hipError_t e, const char *what) {
+  return fail(CCGLIB_ERROR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+  do {                                                  \
+    hipError_t e_ = (expr);                             \
+    if (e_ != hipSuccess) return fail_hip(e_, #expr);   \
+  } while (0)
+
+// Makes `device` current for the lifetime of the guard.
+class DeviceGuard {
+ public:
+  explicit DeviceGuard(int device) {
+    if (hipGetDevice(&previous_) != hipSuccess) previous_ = -1;
+    if (previous_ != device) {
+      status_ = hipSetDevice(device);
+      switched_ = (status_ == hipSuccess);
+    }
+  }
+  ~DeviceGuard() {
+    if (switched_ && previous_ >= 0) (void)hipSetDevice(previous_);
+  }
+  hipError_t status() const { return status_; }
+
+ private:
+  int previous_ = -1;
+  bool switched_ = false;
+  hipError_t status_ = hipSuccess;
+};
+
+int check_device(int device) {
+  int count = 0;
+  HIP_TRY(hipGetDeviceCount(&count));
+  if (device < 0 || device >= count) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "device ordinal %d out of range (%d devices)",
+                device, count);
+  }
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strstr(prop.gcnArchName, "gfx950") == nullptr) {
+    // same wording as the reference's check (src/mma/GEMM.cpp:128-130)
+    return fail(CCGLIB_ERROR_UNSUPPORTED, "This architecture is not supported (%s; need gfx950)",
+                prop.gcnArchName);
+  }
+  return CCGLIB_OK;
+}
+
+bool is_enum01(int v) { return v == 0 || v == 1; }
+
+bool pair_supported(int in, int out) {
+  switch (in) {
+    case kFloat16: return out == kFloat32 || out == kFloat16;
+    case kBfloat16: return out == kFloat32 || out == kBfloat16;
+    case kFloat8e4m3:
+    case kFloat8e5m2: return out == kFloat32;
+    case kInt1: return out == kInt32;
+    default: return false;
+  }
+}
+
+}  // namespace
+
+struct ccglib_gemm {
+  size_t B, M, N, K;
+  int device;
+  hipStream_t stream;
+  int type_in, type_out, variant, c_axis, c_order;
+  float alpha_re, alpha_im, beta_re, beta_im;
+};
+
+struct ccglib_transpose {
+  size_t B, M, N, M_chunk, N_chunk, nr_bits;
+  int device;
+  hipStream_t stream;
+  int axis;
+  size_t input_bytes() const { return B * 2 * M * N * nr_bits / 8; }
+};
+
+struct ccglib_packing {
+  size_t N;
+  int direction, device, axis;
+  hipStream_t stream;
+};
+
+struct ccglib_pipeline {
+  size_t B, M, N, K;
+  int device;
+  hipStream_t stream;
+  int type_in, type_out, c_axis;
+  bool need_copyin_c;
+  ccglib_packing_t pack_a = nullptr, pack_b = nullptr;
+  ccglib_transpose_t trans_a = nullptr, trans_b = nullptr;
+  ccglib_gemm_t gemm = nullptr;
+  void *d_a_packed = nullptr, *d_b_packed = nullptr, *d_a_trans = nullptr, *d_b_trans = nullptr;
+};
+
+extern "C" {
+
+const char *ccglib_last_error(void) { return g_last_error.c_str(); }
+
+const char *ccglib_version(void) { return "ccglib-amd 0.1.0 (gfx950)"; }
+
+/* ------------------------------- GEMM ---------------------------------- */
+
+int ccglib_gemm_get_dimensions(int type_in, int type_out, int variant, unsigned *m_per_block,
+                               unsigned *n_per_block, unsigned *k_chunk) {
+  (void)variant;  // as in the reference, both variants report the same tiles
+  if (!m_per_block || !n_per_block || !k_chunk) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null output pointer");
+  }
+  if (!pair_supported(type_in, type_out)) {
+    // wording of src/mma/Kernel.cpp:38-40
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "No kernel parameters available for selected precision (in %d, out %d)", type_in,
+                type_out);
+  }
+  *m_per_block = kTileRows;
+  *n_per_block = kTileRows;
+  *k_chunk = (unsigned)k_per_tile(type_in);
+  return CCGLIB_OK;
+}
+
+int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t K, int device,
+                       void *stream, int type_in, int type_out, int variant,
+                       int c_complex_axis_location, int c_mem_order, int a_mem_order,
+                       int b_mem_order, float alpha_re, float alpha_im, float beta_re,
+                       float beta_im) {
+  if (!gemm) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
+  *gemm = nullptr;
+  if (!is_enum01(variant) || !is_enum01(c_complex_axis_location) || !is_enum01(c_mem_order) ||
+      !is_enum01(a_mem_order) || !is_enum01(b_mem_order)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  if (variant == kBasic && c_complex_axis_location == kInterleaved) {
+    // src/mma/GEMM.cpp:77-80
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "complex-interleaved output is not supported in basic variant");
+  }
+  if (!pair_supported(type_in, type_out)) {
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "No kernel parameters available for selected precision (in %d, out %d)", type_in,
+                type_out);
+  }
+  if (a_mem_order != kRowMajor || b_mem_order != kColMajor) {
+    // The reference rejects these layouts when it compiles its kernel at
+    // construction (kernels/gemm_kernel_float.cu:20-25); callers match on the
+    // name of that failure (test/gemm/mma.cpp:598-627).
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "HIPRTC_ERROR_COMPILATION: GEMM supports only a row-major A matrix and a "
+                "col-major B matrix");
+  }
+  if (B > 0xffffffffu || M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "problem size out of range");
+  }
+  if (int rc = check_device(device)) return rc;
+  ccglib_gemm *g = new (std::nothrow) ccglib_gemm;
+  if (!g) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
+  g->B = B;
+  g->M = M;
+  g->N = N;
+  g->K = K;
+  g->device = device;
+  g->stream = static_cast<hipStream_t>(stream);
+  g->type_in = type_in;
+  g->type_out = type_out;
+  g->variant = variant;
+  g->c_axis = c_complex_axis_location;
+  g->c_order = c_mem_order;
+  g->alpha_re = alpha_re;
+  g->alpha_im = alpha_im;
+  g->beta_re = beta_re;
+  g->beta_im = beta_im;
+  *gemm = g;
+  return CCGLIB_OK;
+}
+
+int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c) {
+  if (!g) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null GEMM handle");
+  if (g->B == 0 || g->M == 0 || g->N == 0) return CCGLIB_OK;
+  if (!d_a || !d_b || !d_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  GemmParams p;
+  // C[m][n] = sum_k A[m][k] B[n][k]. The kernel wants the operand of the
+  // contiguous C axis as X: B for a row-major C, A for a column-major C (the
+  // complex product commutes, so exchanging the operands transposes C).
+  const bool row_major = (g->c_order == kRowMajor);
+  p.x = row_major ? d_b : d_a;
+  p.y = row_major ? d_a : d_b;
+  p.nx = (unsigned)(row_major ? g->N : g->M);
+  p.ny = (unsigned)(row_major ? g->M : g->N);
+  p.c = d_c;
+  p.batch = (unsigned)g->B;
+  p.k = (unsigned)g->K;
+  p.k_tiles = (unsigned)ceil_div(g->K, (size_t)k_per_tile(g->type_in));
+  if (p.k_tiles == 0) p.k_tiles = 1;  // K = 0: one all-zero tile keeps the epilogue uniform
+  p.x_tiles = (unsigned)ceil_div(p.nx, kTileRows);
+  p.y_tiles = (unsigned)ceil_div(p.ny, kTileRows);
+  p.type_in = g->type_in;
+  p.type_out = g->type_out;
+  p.variant = g->variant;
+  p.c_interleaved = (g->c_axis == kInterleaved);
+  p.alpha_re = g->alpha_re;
+  p.alpha_im = g->alpha_im;
+  p.beta_re = g->beta_re;
+  p.beta_im = g->beta_im;
+  // same switches as the reference's HAVE_ALPHA / HAVE_BETA (src/mma/GEMM.cpp:207-213)
+  p.have_alpha = (g->alpha_re != 1.0f || g->alpha_im != 0.0f);
+  p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
+  if (g->K == 0 && g->variant == kOpt) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "K = 0 has no tiled layout");
+  }
+  DeviceGuard guard(g->device);
+  HIP_TRY(guard.status());
+  const hipError_t e = (g->type_in == kInt1) ? launch_gemm_int1(p, g->stream)
+                                              : launch_gemm_mfma(p, g->stream);
+  if (e != hipSuccess) return fail_hip(e, "GEMM kernel launch");
+  return CCGLIB_OK;
+}
+
+int ccglib_gemm_destroy(ccglib_gemm_t g) {
+  delete g;
+  return CCGLIB_OK;
+}
+
+/* ----------------------------- Transpose -------------------------------- */
+
+int ccglib_transpose_create(ccglib_transpose_t *transpose, size_t B, size_t M, size_t N,
+                            size_t M_chunk, size_t N_chunk, size_t nr_bits, int device,
+                            void *stream, int input_complex_axis_location) {
+  if (!transpose) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
+  *transpose = nullptr;
+  if (!is_enum01(input_complex_axis_location)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  if (nr_bits != 1 && nr_bits != 8 && nr_bits != 16 && nr_bits != 32) {
+    // kernels/transpose_kernel.cu:20-32
+    return fail(CCGLIB_ERROR_UNSUPPORTED, "NBIT_IN must be 1, 8, 16, 32 (got %zu)", nr_bits);
+  }
+  if (M_chunk == 0 || N_chunk == 0) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "chunk sizes must be positive");
+  }
+  if (nr_bits == 1 && (N % 32 != 0 || N_chunk % 32 != 0)) {
+    // one-bit samples move as whole 32-bit words (kernels/transpose_kernel.cu:33,57-59)
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "1-bit transpose needs N and N_chunk to be multiples of 32 (got %zu, %zu)", N,
+                N_chunk);
+  }
+  if (int rc = check_device(device)) return rc;
+  ccglib_transpose *t = new (std::nothrow) ccglib_transpose;
+  if (!t) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
+  t->B = B;
+  t->M = M;
+  t->N = N;
+  t->M_chunk = M_chunk;
+  t->N_chunk = N_chunk;
+  t->nr_bits = nr_bits;
+  t->device = device;
+  t->stream = static_cast<hipStream_t>(stream);
+  t->axis = input_complex_axis_location;
+  *transpose = t;
+  return CCGLIB_OK;
+}
+
+int ccglib_transpose_run(ccglib_transpose_t t, const void *d_input, void *d_output) {
+  if (!t) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null transpose handle");
+  if (t->B == 0 || t->M == 0 || t->N == 0) return CCGLIB_OK;
+  if (!d_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  TransposeParams p;
+  p.in = d_input;
+  p.out = d_output;
+  p.batch = t->B;
+  p.m = t->M;
+  p.m_chunk = t->M_chunk;
+  if (t->nr_bits == 1) {
+    p.elem_bytes = 4;
+    p.n = t->N / 32;
+    p.n_chunk = t->N_chunk / 32;
+  } else {
+    p.elem_bytes = (int)(t->nr_bits / 8);
+    p.n = t->N;
+    p.n_chunk = t->N_chunk;
+  }
+  p.interleaved = (t->axis == kInterleaved);
+  DeviceGuard guard(t->device);
+  HIP_TRY(guard.status());
+  const hipError_t e = launch_transpose(p, t->stream);
+  if (e != hipSuccess) return fail_hip(e, "transpose kernel launch");
+  return CCGLIB_OK;
+}
+
+int ccglib_transpose_run_host(ccglib_transpose_t t, const void *h_input, void *d_output) {
+  if (!t) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null transpose handle");
+  if (!h_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pointer");
+  const size_t bytes = t->input_bytes();
+  if (bytes == 0) return CCGLIB_OK;
+  DeviceGuard guard(t->device);
+  HIP_TRY(guard.status());
+  // stream-ordered staging buffer, as src/transpose/Transpose.cpp:51-56
+  void *d_input = nullptr;
+  HIP_TRY(hipMallocAsync(&d_input, bytes, t->stream));
+  hipError_t e = hipMemcpyAsync(d_input, h_input, bytes, hipMemcpyHostToDevice, t->stream);
+  int rc = CCGLIB_OK;
+  if (e != hipSuccess) rc = fail_hip(e, "hipMemcpyAsync");
+  if (rc == CCGLIB_OK) rc = ccglib_transpose_run(t, d_input, d_output);
+  e = hipFreeAsync(d_input, t->stream);
+  if (rc == CCGLIB_OK && e != hipSuccess) rc = fail_hip(e, "hipFreeAsync");
+  return rc;
+}
+
+int ccglib_transpose_destroy(ccglib_transpose_t t) {
+  delete t;
+  return CCGLIB_OK;
+}
+
+/* ------------------------------ Packing --------------------------------- */
+
+int ccglib_packing_create(ccglib_packing_t *packing, size_t N, int direction, int device,
+                          void *stream, int input_complex_axis_location) {
+  if (!packing) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
+  *packing = nullptr;
+  if (!is_enum01(input_complex_axis_location)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  if (direction != kForward && direction != kBackward) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "Unknown packing direction");
+  }
+  if (direction == kBackward && input_complex_axis_location == kInterleaved) {
+    // src/packing/Packing.cpp:49-53
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "complex-interleaved input is not supported in unpacking kernel");
+  }
+  if (direction == kForward && input_complex_axis_location == kInterleaved && N % 2 != 0) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                "complex-interleaved input needs an even number of samples");
+  }
+  if (int rc = check_device(device)) return rc;
+  ccglib_packing *k = new (std::nothrow) ccglib_packing;
+  if (!k) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
+  k->N = N;
+  k->direction = direction;
+  k->device = device;
+  k->axis = input_complex_axis_location;
+  k->stream = static_cast<hipStream_t>(stream);
+  *packing = k;
+  return CCGLIB_OK;
+}
+
+int ccglib_packing_run(ccglib_packing_t k, const void *d_input, void *d_output) {
+  if (!k) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null packing handle");
+  if (k->N == 0) return CCGLIB_OK;
+  if (!d_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  DeviceGuard guard(k->device);
+  HIP_TRY(guard.status());
+  hipError_t e;
+  if (k->direction == kForward) {
+    e = launch_pack_bits(static_cast<const unsigned char *>(d_input),
+                         static_cast<unsigned *>(d_output), k->N, k->axis == kInterleaved,
+                         k->stream);
+  } else {
+    e = launch_unpack_bits(static_cast<const unsigned *>(d_input),
+                           static_cast<unsigned char *>(d_output), k->N, k->stream);
+  }
+  if (e != hipSuccess) return fail_hip(e, "packing kernel launch");
+  return CCGLIB_OK;
+}
+
+int ccglib_packing_run_host(ccglib_packing_t k, const void *h_input, void *d_output) {
+  if (!k) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null packing handle");
+  if (!h_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pointer");
+  // forward: N bytes of samples; backward: ceil(N/32) packed words
+  const size_t bytes = (k->direction == kForward) ? k->N : ceil_div(k->N, 32) * 4;
+  if (bytes == 0) return CCGLIB_OK;
+  DeviceGuard guard(k->device);
+  HIP_TRY(guard.status());
+  void *d_input = nullptr;
+  HIP_TRY(hipMallocAsync(&d_input, bytes, k->stream));
+  hipError_t e = hipMemcpyAsync(d_input, h_input, bytes, hipMemcpyHostToDevice, k->stream);
+  int rc = CCGLIB_OK;
+  if (e != hipSuccess) rc = fail_hip(e, "hipMemcpyAsync");
+  if (rc == CCGLIB_OK) rc = ccglib_packing_run(k, d_input, d_output);
+  e = hipFreeAsync(d_input, k->stream);
+  if (rc == CCGLIB_OK && e != hipSuccess) rc = fail_hip(e, "hipFreeAsync");
+  return rc;
+}
+
+int ccglib_packing_destroy(ccglib_packing_t k) {
+  delete k;
+  return CCGLIB_OK;
+}
+
+/* ------------------------------ Pipeline -------------------------------- */
+
+int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
+  if (!p) return CCGLIB_OK;
+  {
+    DeviceGuard guard(p->device);
+    if (p->d_a_packed) (void)hipFree(p->d_a_packed);
+    if (p->d_b_packed) (void)hipFree(p->d_b_packed);
+    if (p->d_a_trans) (void)hipFree(p->d_a_trans);
+    if (p->d_b_trans) (void)hipFree(p->d_b_trans);
+  }
+  ccglib_packing_destroy(p->pack_a);
+  ccglib_packing_destroy(p->pack_b);
+  ccglib_transpose_destroy(p->trans_a);
+  ccglib_transpose_destroy(p->trans_b);
+  ccglib_gemm_destroy(p->gemm);
+  delete p;
+  return CCGLIB_OK;
+}
+
+int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
+                           int device, void *stream, int input_complex_axis_location,
+                           int output_complex_axis_location, int a_mem_order, int b_mem_order,
+                           int c_mem_order, int input_type, int output_type, int variant,
+                           float alpha_re, float alpha_im, float beta_re, float beta_im) {
+  if (!pipeline) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
+  *pipeline = nullptr;
+  if (!is_enum01(input_complex_axis_location) || !is_enum01(variant)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  ccglib_pipeline *p = new (std::nothrow) ccglib_pipeline;
+  if (!p) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
+  p->B = B;
+  p->M = M;
+  p->N = N;
+  p->K = K;
+  p->device = device;
+  p->stream = static_cast<hipStream_t>(stream);
+  p->type_in = input_type;
+  p->type_out = output_type;
+  p->c_axis = output_complex_axis_location;
+  p->need_copyin_c = (beta_re != 0.0f || beta_im != 0.0f);  // src/pipeline/Pipeline.cpp:138
+  int rc = CCGLIB_OK;
+  const bool packing = (input_type == kInt1);   // src/pipeline/Pipeline.cpp:52
+  const bool transposing = (variant == kOpt);   // :53
+  // Packing already moves all real samples in front of all imaginary ones
+  // (over the whole buffer), so what follows it sees planar data.
+  const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
+  do {
+    if (packing) {
+      const size_t num_a = B * 2 * M * K, num_b = B * 2 * N * K;  // :57-58
+      if ((rc = ccglib_packing_create(&p->pack_a, num_a, kForward, device, stream,
+                                      input_complex_axis_location)))
+        break;
+      if ((rc = ccglib_packing_create(&p->pack_b, num_b, kForward, device, stream,
+                                      input_complex_axis_location)))
+        break;
+      DeviceGuard guard(device);
+      hipError_t e = hipMalloc(&p->d_a_packed, ceil_div(num_a, 32) * 4 + 16);
+      if (e == hipSuccess) e = hipMalloc(&p->d_b_packed, ceil_div(num_b, 32) * 4 + 16);
+      if (e != hipSuccess) {
+        rc = fail_hip(e, "hipMalloc(packed scratch)");
+        break;
+      }
+    }
+    unsigned mb = 0, nb = 0, kc = 0;
+    if ((rc = ccglib_gemm_get_dimensions(input_type, output_type, variant, &mb, &nb, &kc))) break;
+    if (transposing) {
+      const size_t bits = (size_t)bits_of(input_type);
+      if ((rc = ccglib_transpose_create(&p->trans_a, B, M, K, mb, kc, bits, device, stream,
+                                        axis_after_packing)))  // :78-84
+        break;
+      if ((rc = ccglib_transpose_create(&p->trans_b, B, N, K, nb, kc, bits, device, stream,
+                                        axis_after_packing)))
+        break;
+      // padded to whole tiles (:87-96)
+      const size_t mp = ceil_div(M, mb) * mb, np = ceil_div(N, nb) * nb, kp = ceil_div(K, kc) * kc;
+      DeviceGuard guard(device);
+      hipError_t e = hipMalloc(&p->d_a_trans, B * 2 * mp * kp * bits / 8 + 16);
+      if (e == hipSuccess) e = hipMalloc(&p->d_b_trans, B * 2 * np * kp * bits / 8 + 16);
+      if (e != hipSuccess) {
+        rc = fail_hip(e, "hipMalloc(transposed scratch)");
+        break;
+      }
+    }
+    rc = ccglib_gemm_create(&p->gemm, B, M, N, K, device, stream, input_type, output_type,
+                            variant, output_complex_axis_location, c_mem_order, a_mem_order,
+                            b_mem_order, alpha_re, alpha_im, beta_re, beta_im);  // :102-105
+  } while (false);
+  if (rc != CCGLIB_OK) {
+    const std::string keep = g_last_error;
+    ccglib_pipeline_destroy(p);
+    g_last_error = keep;
+    return rc;
+  }
+  *pipeline = p;
+  return CCGLIB_OK;
+}
+
+int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, void *d_c) {
+  if (!p) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pipeline handle");
+  int rc;
+  const void *a = d_a, *b = d_b;
+  if (p->pack_a) {  // src/pipeline/Pipeline.cpp:111-114
+    if ((rc = ccglib_packing_run(p->pack_a, a, p->d_a_packed))) return rc;
+    if ((rc = ccglib_packing_run(p->pack_b, b, p->d_b_packed))) return rc;
+    a = p->d_a_packed;
+    b = p->d_b_packed;
+  }
+  if (p->trans_a) {  // :116-121
+    if ((rc = ccglib_transpose_run(p->trans_a, a, p->d_a_trans))) return rc;
+    if ((rc = ccglib_transpose_run(p->trans_b, b, p->d_b_trans))) return rc;
+    a = p->d_a_trans;
+    b = p->d_b_trans;
+  }
+  return ccglib_gemm_run(p->gemm, a, b, d_c);  // :123-125
+}
+
+int ccglib_pipeline_run_host(ccglib_pipeline_t p, const void *h_a, const void *h_b, void *h_c) {
+  if (!p) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pipeline handle");
+  if (!h_a || !h_b || !h_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null host pointer");
+  // input is one byte per sample when packing happens inside the pipeline
+  const size_t in_bits = (p->type_in == kInt1) ? 8 : (size_t)bits_of(p->type_in);
+  const size_t bytes_a = p->B * 2 * p->M * p->K * in_bits / 8;
+  const size_t bytes_b = p->B * 2 * p->N * p->K * in_bits / 8;
+  const size_t bytes_c = p->B * 2 * p->M * p->N * (size_t)bits_of(p->type_out) / 8;
+  if (bytes_c == 0) return CCGLIB_OK;
+  DeviceGuard guard(p->device);
+  HIP_TRY(guard.status());
+  void *d_a = nullptr, *d_b = nullptr, *d_c = nullptr;
+  int rc = CCGLIB_OK;
+  hipError_t e = hipMalloc(&d_a, bytes_a ? bytes_a : 16);
+  if (e == hipSuccess) e = hipMalloc(&d_b, bytes_b ? bytes_b : 16);
+  if (e == hipSuccess) e = hipMalloc(&d_c, bytes_c);
+  if (e == hipSuccess && bytes_a) e = hipMemcpyAsync(d_a, h_a, bytes_a, hipMemcpyHostToDevice, p->stream);
+  if (e == hipSuccess && bytes_b) e = hipMemcpyAsync(d_b, h_b, bytes_b, hipMemcpyHostToDevice, p->stream);
+  if (e == hipSuccess) {
+    // src/pipeline/Pipeline.cpp:168-172
+    e = p->need_copyin_c ? hipMemcpyAsync(d_c, h_c, bytes_c, hipMemcpyHostToDevice, p->stream)
+                         : hipMemsetAsync(d_c, 0, bytes_c, p->stream);
+  }
+  if (e != hipSuccess) rc = fail_hip(e, "pipeline host staging");
+  if (rc == CCGLIB_OK) rc = ccglib_pipeline_run(p, d_a, d_b, d_c);
+  if (rc == CCGLIB_OK) {
+    e = hipMemcpyAsync(h_c, d_c, bytes_c, hipMemcpyDeviceToHost, p->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(p->stream);
+    if (e != hipSuccess) rc = fail_hip(e, "pipeline copy back");
+  } else {
+    (void)hipStreamSynchronize(p->stream);
+  }
+  if (d_a) (void)hipFree(d_a);
+  if (d_b) (void)hipFree(d_b);
+  if (d_c) (void)hipFree(d_c);
+  return rc;
+}
+
+}  // extern "C"

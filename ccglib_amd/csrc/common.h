@@ -1,0 +1,95 @@
+// Shared definitions of the gfx950 complex-GEMM library: enum values, launch
+// parameter blocks handed from the C ABI layer to the kernel launchers, and
+// the tile geometry every kernel agrees on.
+#ifndef CCGLIB_AMD_COMMON_H_
+#define CCGLIB_AMD_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace ccglib_amd {
+
+// Values of the reference enums (include/ccglib/common/value_type.h:14-22).
+enum ValueType : int {
+  kInt1 = 0,
+  kInt32 = 1,
+  kBfloat16 = 2,
+  kFloat8e4m3 = 3,
+  kFloat8e5m2 = 4,
+  kFloat16 = 5,
+  kFloat32 = 6
+};
+enum : int { kPlanar = 0, kInterleaved = 1 };
+enum : int { kForward = 0, kBackward = 1 };
+enum : int { kRowMajor = 0, kColMajor = 1 };
+enum : int { kBasic = 0, kOpt = 1 };
+
+// Tile geometry of the optimised layout. Every operand tile is 128 rows of
+// 64 bytes of K (32 half/bfloat16 values, 64 fp8 values or 512 one-bit
+// samples), real plane then imaginary plane: 16 KiB that are contiguous in
+// memory, so a block copies a tile into LDS with plain 16-byte loads.
+constexpr int kTileRows = 128;
+constexpr int kTileRowBytes = 64;
+constexpr int kTilePlaneBytes = kTileRows * kTileRowBytes;  // 8 KiB
+constexpr int kTileBytes = 2 * kTilePlaneBytes;             // 16 KiB
+
+inline size_t ceil_div(size_t a, size_t b) { return a / b + (a % b != 0); }
+
+inline int bits_of(int type) {
+  switch (type) {
+    case kInt1: return 1;
+    case kFloat8e4m3:
+    case kFloat8e5m2: return 8;
+    case kBfloat16:
+    case kFloat16: return 16;
+    case kFloat32:
+    case kInt32: return 32;
+    default: return 0;
+  }
+}
+
+// K values (samples) held by one 64-byte tile row.
+inline int k_per_tile(int type_in) { return kTileRowBytes * 8 / bits_of(type_in); }
+
+// Problem description for one GEMM launch, in kernel terms. The kernel
+// computes D[y][x] = sum_k X[x][k] * Y[y][k] with x the contiguous output
+// axis: for a row-major C, X is the caller's B (N rows) and Y the caller's A
+// (M rows); for a column-major C the two are exchanged by the host, which is
+// valid because the complex product commutes.
+struct GemmParams {
+  const void *x;        // operand whose rows index the contiguous C axis
+  const void *y;        // operand whose rows index the strided C axis
+  void *c;
+  unsigned batch;
+  unsigned nx, ny;      // logical (un-padded) rows of X and Y
+  unsigned k;           // logical K in samples
+  unsigned k_tiles;     // number of 64-byte K tiles (ceil)
+  unsigned x_tiles, y_tiles;  // 128-row tiles per operand (ceil)
+  int type_in, type_out;
+  int variant;          // kBasic: planar rows; kOpt: tiled layout
+  int c_interleaved;    // 0 planar, 1 interleaved
+  float alpha_re, alpha_im, beta_re, beta_im;
+  int have_alpha, have_beta;
+};
+
+hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream);
+hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream);
+
+struct TransposeParams {
+  const void *in;
+  void *out;
+  size_t batch, m, n;        // n in elements of elem_bytes (words for 1 bit)
+  size_t m_chunk, n_chunk;   // likewise
+  int elem_bytes;            // 1, 2 or 4
+  int interleaved;
+};
+hipError_t launch_transpose(const TransposeParams &p, hipStream_t stream);
+
+hipError_t launch_pack_bits(const unsigned char *in, unsigned *out, size_t n,
+                            int interleaved, hipStream_t stream);
+hipError_t launch_unpack_bits(const unsigned *in, unsigned char *out, size_t n,
+                              hipStream_t stream);
+
+}  // namespace ccglib_amd
+#endif  // CCGLIB_AMD_COMMON_H_

@@ -1,0 +1,171 @@
+// Device-side helpers shared by the complex GEMM kernels: the LDS swizzle, the
+// operand loaders for the tiled and the planar layouts, the kernel argument
+// block and the workgroup-to-tile mapping.
+#ifndef CCGLIB_AMD_GEMM_DEVICE_H_
+#define CCGLIB_AMD_GEMM_DEVICE_H_
+
+#include "common.h"
+
+namespace ccglib_amd {
+
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+enum Loader { kLoadTiled = 0, kLoadPlanarVec = 1, kLoadPlanarElem = 2 };
+
+constexpr int kNumXcd = 8;
+
+// LDS rows are 64 bytes; XORing the 16-byte chunk index with (row >> 1) & 3
+// keeps linear 16-byte writes and 16-row column reads free of bank conflicts.
+__device__ __forceinline__ int swizzled_row_offset(int row, int chunk) {
+  return row * kTileRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4);
+}
+
+// Description of one operand as the loader sees it.
+struct OperandView {
+  const char *base;   // start of this batch's data
+  unsigned rows;      // logical rows
+  unsigned tiles;     // 128-row tiles (tiled layout)
+  unsigned row0;      // first row of this block
+};
+
+// Loads the 16-byte chunk (k tile kt, plane, row, chunk c) of an operand.
+// Out-of-range chunks read a clamped, valid address and are then replaced by
+// zero, so the vector paths issue their loads without branches.
+template <int EB, int LOADER>
+__device__ __forceinline__ int4_t load_chunk(const OperandView &op, unsigned kt, unsigned k_tiles,
+                                             unsigned k_bytes, int plane, int row, int c) {
+  const int4_t zero = {0, 0, 0, 0};
+  const unsigned grow = op.row0 + row;
+  if constexpr (LOADER == kLoadTiled) {
+    const unsigned tile = grow / kTileRows;
+    const bool valid = (kt < k_tiles) && (tile < op.tiles);
+    const unsigned tile_c = tile < op.tiles ? tile : op.tiles - 1;
+    const unsigned kt_c = kt < k_tiles ? kt : k_tiles - 1;
+    const size_t off = ((size_t)tile_c * k_tiles + kt_c) * kTileBytes + plane * kTilePlaneBytes +
+                       (grow % kTileRows) * kTileRowBytes + c * 16;
+    const int4_t v = *reinterpret_cast<const int4_t *>(op.base + off);
+    return valid ? v : zero;
+  } else {
+    const unsigned kb = kt * kTileRowBytes + c * 16;
+    if constexpr (LOADER == kLoadPlanarVec) {
+      const bool valid = (grow < op.rows) && (kb + 16 <= k_bytes);
+      const unsigned row_c = grow < op.rows ? grow : op.rows - 1;
+      const unsigned kb_c = (kb + 16 <= k_bytes) ? kb : 0;
+      const char *p = op.base + ((size_t)plane * op.rows + row_c) * k_bytes + kb_c;
+      const int4_t v = *reinterpret_cast<const int4_t *>(p);
+      return valid ? v : zero;
+    } else {
+      int4_t v = zero;
+      if (grow >= op.rows || kb >= k_bytes) return v;
+      const char *p = op.base + ((size_t)plane * op.rows + grow) * k_bytes + kb;
+      if constexpr (EB == 2) {
+        const unsigned short *q = reinterpret_cast<const unsigned short *>(p);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          unsigned s = (kb + 2 * e < k_bytes) ? q[e] : 0u;
+          v[e / 2] |= (int)(s << (16 * (e % 2)));
+        }
+      } else if constexpr (EB == 4) {
+        const unsigned *q = reinterpret_cast<const unsigned *>(p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = (kb + 4 * e < k_bytes) ? (int)q[e] : 0;
+        }
+      } else {
+        const unsigned char *q = reinterpret_cast<const unsigned char *>(p);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          unsigned s = (kb + e < k_bytes) ? q[e] : 0u;
+          v[e / 4] |= (int)(s << (8 * (e % 4)));
+        }
+      }
+      return v;
+    }
+  }
+}
+
+struct KernelArgs {
+  const char *x;
+  const char *y;
+  char *c;
+  unsigned batch, nx, ny, k, k_tiles, k_bytes, x_tiles, y_tiles;
+  unsigned blocks_x, blocks_y;
+  size_t x_batch_bytes, y_batch_bytes;
+  float alpha_re, alpha_im, beta_re, beta_im;
+  int have_alpha, have_beta, c_interleaved;
+};
+
+// Maps the hardware workgroup id to a logical tile id such that the ids that
+// one XCD receives (every 8th workgroup) are consecutive.
+__device__ __forceinline__ unsigned xcd_remap(unsigned wg, unsigned total) {
+  const unsigned xcd = wg % kNumXcd;
+  const unsigned idx = wg / kNumXcd;
+  const unsigned q = total / kNumXcd, r = total % kNumXcd;
+  const unsigned start = xcd * q + (xcd < r ? xcd : r);
+  return start + idx;
+}
+
+
+// Splits the logical tile id into (batch, block_x, block_y). Inside a batch,
+// tiles are walked in groups of 4 block rows with y fastest, so the 32
+// consecutive tiles that one XCD works on touch 4 Y panels and 8 X panels.
+struct TileCoord {
+  unsigned b, block_x, block_y;
+};
+__device__ __forceinline__ TileCoord tile_coord(const KernelArgs &args, unsigned wg) {
+  const unsigned per_batch = args.blocks_x * args.blocks_y;
+  const unsigned logical = xcd_remap(wg, per_batch * args.batch);
+  TileCoord tc;
+  tc.b = logical / per_batch;
+  unsigned t = logical % per_batch;
+  constexpr unsigned GROUP = 4;
+  const unsigned group_size = GROUP * args.blocks_x;
+  const unsigned g = t / group_size;
+  const unsigned first_y = g * GROUP;
+  const unsigned rows_in_group =
+      (args.blocks_y - first_y) < GROUP ? (args.blocks_y - first_y) : GROUP;
+  t -= g * group_size;
+  tc.block_y = first_y + t % rows_in_group;
+  tc.block_x = t / rows_in_group;
+  return tc;
+}
+
+// Fills the kernel argument block from the launch parameters for a BX x BY
+// block tile.
+inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
+  KernelArgs a;
+  a.x = static_cast<const char *>(p.x);
+  a.y = static_cast<const char *>(p.y);
+  a.c = static_cast<char *>(p.c);
+  a.batch = p.batch;
+  a.nx = p.nx;
+  a.ny = p.ny;
+  a.k = p.k;
+  a.k_tiles = p.k_tiles;
+  // bytes of K per row of a planar operand: 1-bit samples are stored in whole
+  // 32-bit words
+  a.k_bytes = (p.type_in == kInt1) ? (unsigned)(ceil_div(p.k, 32) * 4)
+                                   : (unsigned)((size_t)p.k * bits_of(p.type_in) / 8);
+  a.x_tiles = p.x_tiles;
+  a.y_tiles = p.y_tiles;
+  a.blocks_x = (unsigned)ceil_div(p.nx, bx);
+  a.blocks_y = (unsigned)ceil_div(p.ny, by);
+  if (p.variant == kOpt) {
+    a.x_batch_bytes = (size_t)p.x_tiles * p.k_tiles * kTileBytes;
+    a.y_batch_bytes = (size_t)p.y_tiles * p.k_tiles * kTileBytes;
+  } else {
+    a.x_batch_bytes = (size_t)2 * p.nx * a.k_bytes;
+    a.y_batch_bytes = (size_t)2 * p.ny * a.k_bytes;
+  }
+  a.alpha_re = p.alpha_re;
+  a.alpha_im = p.alpha_im;
+  a.beta_re = p.beta_re;
+  a.beta_im = p.beta_im;
+  a.have_alpha = p.have_alpha;
+  a.have_beta = p.have_beta;
+  a.c_interleaved = p.c_interleaved;
+  return a;
+}
+
+}  // namespace ccglib_amd
+#endif  // CCGLIB_AMD_GEMM_DEVICE_H_

@@ -1,0 +1,386 @@
+// Complex GEMM on the gfx950 matrix cores for fp16, bf16 and fp8 (e4m3/e5m2)
+// input with fp32 accumulation.
+//
+// Stands in for the reference's wmma_complex_gemm_basic / wmma_complex_gemm_opt
+// (kernels/gemm_kernel_float.cu:35-181, :186-355) and its epilogue helpers
+// (kernels/matrix_operations.h:38-178). The math is the same four real
+// products per complex product (gemm_kernel_float.cu:293-303); everything
+// else is laid out for 64-wide wavefronts:
+//
+//  * One block owns a BX x BY patch of C and walks K in stages of KT tiles of
+//    64 bytes. Operand tiles are staged global -> registers -> LDS one stage
+//    ahead of the math (two LDS stages, one barrier per stage).
+//  * LDS rows are 64 bytes; the 16-byte chunk index is XORed with
+//    (row >> 1) & 3, which makes both the linear 16-byte writes and the
+//    16-row fragment reads free of bank conflicts on this LDS.
+//  * 16x16x32 MFMA (16x16x128 for fp8). The operand whose rows run along the
+//    contiguous axis of C is the MFMA "A" operand, so each lane ends up with
+//    four consecutive C elements and stores them with one 16-byte write.
+//  * The four products of a complex MAC reuse the same fragments; the minus
+//    sign of Re -= Xi*Yi is a sign-bit flip of the Yi fragment registers.
+//  * Workgroup ids are remapped so that consecutive tiles land on the same
+//    XCD (shared L2), in groups that reuse both operands.
+#include "gemm_device.h"
+
+namespace ccglib_amd {
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef int int8_t_ __attribute__((ext_vector_type(8)));
+typedef unsigned short ushort4_t __attribute__((ext_vector_type(4)));
+
+// K tiles consumed by one MFMA: one for 16-bit input (16x16x32), two for fp8
+// (16x16x128: 32 bytes per lane, 16 from each of two K tiles).
+template <int DT> struct DtypeTraits {
+  static constexpr int kTilesPerMfma = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 2 : 1;
+  static constexpr int kElemBytes = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 1 : 2;
+  static constexpr unsigned kSignMask =
+      (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u : 0x80008000u;
+};
+
+template <int DT> struct Fragment {
+  int4_t v[DtypeTraits<DT>::kTilesPerMfma];
+};
+
+template <int DT>
+__device__ __forceinline__ float4_t mfma(const Fragment<DT> &a, const Fragment<DT> &b,
+                                         float4_t acc) {
+  if constexpr (DT == kFloat16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+        __builtin_bit_cast(half8_t, a.v[0]), __builtin_bit_cast(half8_t, b.v[0]), acc, 0, 0, 0);
+  } else if constexpr (DT == kBfloat16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(bf16x8_t, a.v[0]), __builtin_bit_cast(bf16x8_t, b.v[0]), acc, 0, 0, 0);
+  } else {
+    int8_t_ av, bv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      av[i] = a.v[0][i];
+      av[4 + i] = a.v[1][i];
+      bv[i] = b.v[0][i];
+      bv[4 + i] = b.v[1][i];
+    }
+    // format code 0 = e4m3, 1 = e5m2; scale exponent 127 = 2^0
+    constexpr int fmt = (DT == kFloat8e4m3) ? 0 : 1;
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc, fmt, fmt, 0, 0x7f, 0,
+                                                            0x7f);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ Fragment<DT> negate(const Fragment<DT> &f) {
+  Fragment<DT> r;
+#pragma unroll
+  for (int t = 0; t < DtypeTraits<DT>::kTilesPerMfma; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      r.v[t][i] = f.v[t][i] ^ (int)DtypeTraits<DT>::kSignMask;
+    }
+  }
+  return r;
+}
+
+template <int TOUT> struct OutType;
+template <> struct OutType<kFloat32> { using type = float; };
+template <> struct OutType<kFloat16> { using type = _Float16; };
+template <> struct OutType<kBfloat16> { using type = __bf16; };
+
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WAVES_PER_EU>
+__global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma(
+    const KernelArgs args) {
+  using Tout = typename OutType<TOUT>::type;
+  constexpr int NWX = BX / WX, NWY = BY / WY;
+  constexpr int NTHREADS = 64 * NWX * NWY;
+  constexpr int TX = WX / 16, TY = WY / 16;
+  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  static_assert(KT % KPM == 0, "stage must hold whole MFMAs");
+  constexpr int X_KTILE_BYTES = 2 * BX * kTileRowBytes;
+  constexpr int Y_KTILE_BYTES = 2 * BY * kTileRowBytes;
+  constexpr int KTILE_BYTES = X_KTILE_BYTES + Y_KTILE_BYTES;
+  constexpr int STAGE_BYTES = KT * KTILE_BYTES;
+  constexpr int X_CHUNKS = KT * 2 * BX * 4;
+  constexpr int Y_CHUNKS = KT * 2 * BY * 4;
+  static_assert(X_CHUNKS % NTHREADS == 0 && Y_CHUNKS % NTHREADS == 0, "chunks per thread");
+  constexpr int CX = X_CHUNKS / NTHREADS, CY = Y_CHUNKS / NTHREADS;
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wx = wave % NWX, wy = wave / NWX;
+
+  // ---- which tile of C -------------------------------------------------
+  const TileCoord tc = tile_coord(args, blockIdx.x);
+  const unsigned b = tc.b, block_x = tc.block_x, block_y = tc.block_y;
+
+  OperandView xv{args.x + (size_t)b * args.x_batch_bytes, args.nx, args.x_tiles, block_x * BX};
+  OperandView yv{args.y + (size_t)b * args.y_batch_bytes, args.ny, args.y_tiles, block_y * BY};
+  const unsigned k_tiles = args.k_tiles;
+  const unsigned k_bytes = args.k_bytes;
+
+  // ---- staging registers and their LDS destinations --------------------
+  int4_t xs[CX], ys[CY];
+  auto fetch = [&](unsigned kt0) {
+#pragma unroll
+    for (int i = 0; i < CX; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
+      xs[i] = load_chunk<DtypeTraits<DT>::kElemBytes, LOADER>(
+          xv, kt0 + kk, k_tiles, k_bytes, rem / (BX * 4), (rem / 4) % BX, rem % 4);
+    }
+#pragma unroll
+    for (int i = 0; i < CY; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
+      ys[i] = load_chunk<DtypeTraits<DT>::kElemBytes, LOADER>(
+          yv, kt0 + kk, k_tiles, k_bytes, rem / (BY * 4), (rem / 4) % BY, rem % 4);
+    }
+  };
+  auto stash = [&](int stage) {
+    char *s = lds + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < CX; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
+      const int plane = rem / (BX * 4), row = (rem / 4) % BX, c = rem % 4;
+      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + plane * BX * kTileRowBytes +
+                                  swizzled_row_offset(row, c)) = xs[i];
+    }
+#pragma unroll
+    for (int i = 0; i < CY; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
+      const int plane = rem / (BY * 4), row = (rem / 4) % BY, c = rem % 4;
+      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + X_KTILE_BYTES +
+                                  plane * BY * kTileRowBytes + swizzled_row_offset(row, c)) =
+          ys[i];
+    }
+  };
+
+  // ---- accumulators ------------------------------------------------------
+  float4_t acc_re[TY][TX], acc_im[TY][TX];
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+#pragma unroll
+    for (int i = 0; i < TX; ++i) {
+      acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  const int lane_off = swizzled_row_offset(lane & 15, lane >> 4);
+  const int x_frag_base = (wx * WX) * kTileRowBytes + lane_off;
+  const int y_frag_base = X_KTILE_BYTES + (wy * WY) * kTileRowBytes + lane_off;
+
+  auto compute = [&](int stage) {
+    const char *s = lds + stage * STAGE_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < KT; kk += KPM) {
+      Fragment<DT> xr[TX], xi[TX];
+#pragma unroll
+      for (int i = 0; i < TX; ++i) {
+#pragma unroll
+        for (int u = 0; u < KPM; ++u) {
+          const char *p = s + (kk + u) * KTILE_BYTES + x_frag_base + i * 16 * kTileRowBytes;
+          xr[i].v[u] = *reinterpret_cast<const int4_t *>(p);
+          xi[i].v[u] = *reinterpret_cast<const int4_t *>(p + BX * kTileRowBytes);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TY; ++j) {
+        Fragment<DT> yr, yi;
+#pragma unroll
+        for (int u = 0; u < KPM; ++u) {
+          const char *p = s + (kk + u) * KTILE_BYTES + y_frag_base + j * 16 * kTileRowBytes;
+          yr.v[u] = *reinterpret_cast<const int4_t *>(p);
+          yi.v[u] = *reinterpret_cast<const int4_t *>(p + BY * kTileRowBytes);
+        }
+        const Fragment<DT> yin = negate<DT>(yi);
+#pragma unroll
+        for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xr[i], yr, acc_re[j][i]);
+#pragma unroll
+        for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xr[i], yi, acc_im[j][i]);
+#pragma unroll
+        for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
+#pragma unroll
+        for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
+      }
+    }
+  };
+
+  // ---- main loop ---------------------------------------------------------
+  const unsigned stages = (k_tiles + KT - 1) / KT;
+  fetch(0);
+  stash(0);
+  if (stages > 1) fetch(KT);
+  __syncthreads();
+  for (unsigned s = 0; s < stages; ++s) {
+    const int cur = s & 1;
+    if (s + 1 < stages) stash(cur ^ 1);
+    if (s + 2 < stages) fetch((s + 2) * KT);
+    compute(cur);
+    __syncthreads();
+  }
+
+  // ---- epilogue: alpha * acc + beta * C, store ---------------------------
+  // lane holds, per 16x16 tile, x = x0 + (lane/16)*4 + 0..3 at y = y0 + lane%16
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha, have_beta = args.have_beta;
+  const float ar = args.alpha_re, ai = args.alpha_im, br = args.beta_re, bi = args.beta_im;
+  Tout *cbase = reinterpret_cast<Tout *>(args.c) + (size_t)b * 2 * nx * ny;
+  const bool vec_ok = (nx % 4 == 0);
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+    const unsigned y = block_y * BY + wy * WY + j * 16 + (lane & 15);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) {
+      const unsigned x = block_x * BX + wx * WX + i * 16 + (lane >> 4) * 4;
+      if (y >= ny || x >= nx) continue;
+      float re[4], im[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        re[e] = acc_re[j][i][e];
+        im[e] = acc_im[j][i][e];
+        if (have_alpha) {
+          const float r0 = re[e];
+          re[e] = ar * r0 - ai * im[e];
+          im[e] = ai * r0 + ar * im[e];
+        }
+      }
+      const bool full = vec_ok && (x + 4 <= nx);
+      if (!args.c_interleaved) {
+        Tout *pr = cbase + (size_t)y * nx + x;
+        Tout *pi = pr + (size_t)nx * ny;
+        if (have_beta) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              const float cr = (float)pr[e], ci = (float)pi[e];
+              re[e] += br * cr - bi * ci;
+              im[e] += bi * cr + br * ci;
+            }
+          }
+        }
+        if (full) {
+          if constexpr (TOUT == kFloat32) {
+            *reinterpret_cast<float4_t *>(pr) = float4_t{re[0], re[1], re[2], re[3]};
+            *reinterpret_cast<float4_t *>(pi) = float4_t{im[0], im[1], im[2], im[3]};
+          } else {
+            Tout r4[4] = {(Tout)re[0], (Tout)re[1], (Tout)re[2], (Tout)re[3]};
+            Tout i4[4] = {(Tout)im[0], (Tout)im[1], (Tout)im[2], (Tout)im[3]};
+            *reinterpret_cast<ushort4_t *>(pr) = __builtin_bit_cast(ushort4_t, r4);
+            *reinterpret_cast<ushort4_t *>(pi) = __builtin_bit_cast(ushort4_t, i4);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              pr[e] = (Tout)re[e];
+              pi[e] = (Tout)im[e];
+            }
+          }
+        }
+      } else {
+        Tout *p = cbase + ((size_t)y * nx + x) * 2;
+        if (have_beta) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              const float cr = (float)p[2 * e], ci = (float)p[2 * e + 1];
+              re[e] += br * cr - bi * ci;
+              im[e] += bi * cr + br * ci;
+            }
+          }
+        }
+        if (full) {
+          if constexpr (TOUT == kFloat32) {
+            reinterpret_cast<float4_t *>(p)[0] = float4_t{re[0], im[0], re[1], im[1]};
+            reinterpret_cast<float4_t *>(p)[1] = float4_t{re[2], im[2], re[3], im[3]};
+          } else {
+            Tout v8[8] = {(Tout)re[0], (Tout)im[0], (Tout)re[1], (Tout)im[1],
+                          (Tout)re[2], (Tout)im[2], (Tout)re[3], (Tout)im[3]};
+            *reinterpret_cast<int4_t *>(p) = __builtin_bit_cast(int4_t, v8);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              p[2 * e] = (Tout)re[e];
+              p[2 * e + 1] = (Tout)im[e];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WPE>
+hipError_t launch_config(const GemmParams &p, hipStream_t stream) {
+  constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
+  constexpr int LDS_BYTES = 2 * KT * 2 * (BX + BY) * kTileRowBytes;
+  const KernelArgs a = make_kernel_args(p, BX, BY);
+  const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
+  if (total == 0) return hipSuccess;
+  if (total > 0x7fffffffu) return hipErrorInvalidValue;
+  auto kernel = complex_gemm_mfma<DT, TOUT, BX, BY, WX, WY, KT, LOADER, WPE>;
+  if (LDS_BYTES > 64 * 1024) {
+    static bool raised = false;  // per instantiation
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+      if (e != hipSuccess) return e;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(NTHREADS), LDS_BYTES, stream, a);
+  return hipGetLastError();
+}
+
+template <int DT, int TOUT>
+hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
+  constexpr int KT = DtypeTraits<DT>::kTilesPerMfma;
+  // fp8 stages are twice as large (two K tiles per MFMA): one block per CU,
+  // one wave per SIMD with the full register file
+  constexpr int WPE = (KT == 2) ? 1 : 2;
+  if (p.variant == kOpt) {
+    return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadTiled, WPE>(p, stream);
+  }
+  const size_t k_bytes = (size_t)p.k * bits_of(p.type_in) / 8;
+  const bool aligned = (k_bytes >= 16) && (k_bytes % 16 == 0) && ((uintptr_t)p.x % 16 == 0) &&
+                       ((uintptr_t)p.y % 16 == 0);
+  if (aligned) {
+    return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadPlanarVec, WPE>(p, stream);
+  }
+  return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadPlanarElem, WPE>(p, stream);
+}
+
+}  // namespace
+
+hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
+  switch (p.type_in) {
+    case kFloat16:
+      if (p.type_out == kFloat32) return launch_typed<kFloat16, kFloat32>(p, stream);
+      if (p.type_out == kFloat16) return launch_typed<kFloat16, kFloat16>(p, stream);
+      break;
+    case kBfloat16:
+      if (p.type_out == kFloat32) return launch_typed<kBfloat16, kFloat32>(p, stream);
+      if (p.type_out == kBfloat16) return launch_typed<kBfloat16, kBfloat16>(p, stream);
+      break;
+    case kFloat8e4m3:
+      if (p.type_out == kFloat32) return launch_typed<kFloat8e4m3, kFloat32>(p, stream);
+      break;
+    case kFloat8e5m2:
+      if (p.type_out == kFloat32) return launch_typed<kFloat8e5m2, kFloat32>(p, stream);
+      break;
+    default:
+      break;
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace ccglib_amd

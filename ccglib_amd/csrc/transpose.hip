@@ -1,0 +1,185 @@
+// Transpose into the tiled layout of the optimised GEMM:
+//   in  [B][2][M][N] (planar) or [B][M][N][2] (interleaved)
+//   out [B][Mp/Mc][Np/Nc][2][Mc][Nc], zero where m >= M or n >= N.
+// Stands in for the reference's transpose kernel
+// (kernels/transpose_kernel.cu:50-82), which moves one element pair per
+// thread. This one is bandwidth-shaped: a thread moves 16-byte vectors (both
+// planes of 4 rows), lanes of a wave run along N across tile boundaries, so
+// loads are contiguous runs of 256 bytes per row and stores are contiguous
+// runs of rows inside each output tile. A scalar kernel covers shapes whose
+// rows are not whole 16-byte vectors.
+#include "common.h"
+
+namespace ccglib_amd {
+namespace {
+
+typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+typedef unsigned short ushort8_t __attribute__((ext_vector_type(8)));
+typedef unsigned char uchar16_t __attribute__((ext_vector_type(16)));
+
+struct TransposeArgs {
+  const char *in;
+  char *out;
+  size_t m, n;              // logical sizes in elements
+  size_t m_chunk, n_chunk;  // tile sizes in elements
+  size_t m_tiles, n_tiles;
+  size_t n_vecs_padded;     // 16-byte vectors per padded row
+  size_t vecs_per_tile_row;
+};
+
+// De-interleaves two 16-byte vectors holding (re, im) pairs.
+template <int EB>
+__device__ __forceinline__ void deinterleave(uint4_t a, uint4_t b, uint4_t &re, uint4_t &im) {
+  if constexpr (EB == 4) {
+    re = uint4_t{a[0], a[2], b[0], b[2]};
+    im = uint4_t{a[1], a[3], b[1], b[3]};
+  } else if constexpr (EB == 2) {
+    const ushort8_t x = __builtin_bit_cast(ushort8_t, a), y = __builtin_bit_cast(ushort8_t, b);
+    re = __builtin_bit_cast(uint4_t, __builtin_shufflevector(x, y, 0, 2, 4, 6, 8, 10, 12, 14));
+    im = __builtin_bit_cast(uint4_t, __builtin_shufflevector(x, y, 1, 3, 5, 7, 9, 11, 13, 15));
+  } else {
+    const uchar16_t x = __builtin_bit_cast(uchar16_t, a), y = __builtin_bit_cast(uchar16_t, b);
+    re = __builtin_bit_cast(uint4_t, __builtin_shufflevector(x, y, 0, 2, 4, 6, 8, 10, 12, 14, 16,
+                                                             18, 20, 22, 24, 26, 28, 30));
+    im = __builtin_bit_cast(uint4_t, __builtin_shufflevector(x, y, 1, 3, 5, 7, 9, 11, 13, 15, 17,
+                                                             19, 21, 23, 25, 27, 29, 31));
+  }
+}
+
+constexpr int kRowsPerThread = 4;
+constexpr int kVecsPerBlockRow = 16;   // 256 bytes of a row per block
+constexpr int kRowsPerBlock = 16 * kRowsPerThread;
+
+// grid: (ceil(n_vecs_padded / 16), ceil(Mp / 64), B); block: 256 threads as
+// 16 vectors x 16 rows, each thread doing rows r, r+16, r+32, r+48.
+template <int EB, bool INTERLEAVED>
+__global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
+  constexpr int V = 16 / EB;  // elements per vector
+  const size_t nvec = (size_t)blockIdx.x * kVecsPerBlockRow + (threadIdx.x & 15);
+  const size_t m_base = (size_t)blockIdx.y * kRowsPerBlock + (threadIdx.x >> 4);
+  const size_t b = blockIdx.z;
+  const size_t m_padded = a.m_tiles * a.m_chunk;
+  if (nvec >= a.n_vecs_padded) return;
+  const size_t n0 = nvec * V;
+  const bool n_ok = n0 < a.n;  // rows are whole vectors: inside or outside
+  const size_t nt = nvec / a.vecs_per_tile_row, v = nvec % a.vecs_per_tile_row;
+  const size_t plane_bytes = a.m_chunk * a.n_chunk * EB;
+
+  uint4_t re[kRowsPerThread], im[kRowsPerThread];
+#pragma unroll
+  for (int i = 0; i < kRowsPerThread; ++i) {
+    const size_t m = m_base + 16 * i;
+    re[i] = uint4_t{0, 0, 0, 0};
+    im[i] = uint4_t{0, 0, 0, 0};
+    if (m < a.m && n_ok) {
+      if constexpr (!INTERLEAVED) {
+        const char *p = a.in + (((b * 2) * a.m + m) * a.n + n0) * EB;
+        re[i] = *reinterpret_cast<const uint4_t *>(p);
+        im[i] = *reinterpret_cast<const uint4_t *>(p + a.m * a.n * EB);
+      } else {
+        const char *p = a.in + ((b * a.m + m) * a.n + n0) * 2 * EB;
+        const uint4_t x = *reinterpret_cast<const uint4_t *>(p);
+        const uint4_t y = *reinterpret_cast<const uint4_t *>(p + 16);
+        deinterleave<EB>(x, y, re[i], im[i]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRowsPerThread; ++i) {
+    const size_t m = m_base + 16 * i;
+    if (m < m_padded) {
+      const size_t mt = m / a.m_chunk, mr = m % a.m_chunk;
+      char *q = a.out + (((b * a.m_tiles + mt) * a.n_tiles + nt) * 2) * plane_bytes +
+                (mr * a.n_chunk) * EB + v * 16;
+      *reinterpret_cast<uint4_t *>(q) = re[i];
+      *reinterpret_cast<uint4_t *>(q + plane_bytes) = im[i];
+    }
+  }
+}
+
+// One thread per output element pair; any shape.
+template <typename T, bool INTERLEAVED>
+__global__ __launch_bounds__(256) void transpose_scalar(const TransposeArgs a, size_t batch) {
+  const size_t n_padded = a.n_tiles * a.n_chunk;
+  const size_t m_padded = a.m_tiles * a.m_chunk;
+  const size_t per_batch = m_padded * n_padded;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= per_batch * batch) return;
+  const size_t b = idx / per_batch;
+  const size_t m = (idx % per_batch) / n_padded, n = idx % n_padded;
+  const T *in = reinterpret_cast<const T *>(a.in);
+  T *out = reinterpret_cast<T *>(a.out);
+  T re = 0, im = 0;
+  if (m < a.m && n < a.n) {
+    if constexpr (!INTERLEAVED) {
+      re = in[((b * 2) * a.m + m) * a.n + n];
+      im = in[((b * 2 + 1) * a.m + m) * a.n + n];
+    } else {
+      re = in[((b * a.m + m) * a.n + n) * 2];
+      im = in[((b * a.m + m) * a.n + n) * 2 + 1];
+    }
+  }
+  const size_t mt = m / a.m_chunk, mr = m % a.m_chunk;
+  const size_t nt = n / a.n_chunk, nr = n % a.n_chunk;
+  const size_t plane = a.m_chunk * a.n_chunk;
+  const size_t o = (((b * a.m_tiles + mt) * a.n_tiles + nt) * 2) * plane + mr * a.n_chunk + nr;
+  out[o] = re;
+  out[o + plane] = im;
+}
+
+template <int EB, typename T>
+hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
+  TransposeArgs a;
+  a.in = static_cast<const char *>(p.in);
+  a.out = static_cast<char *>(p.out);
+  a.m = p.m;
+  a.n = p.n;
+  a.m_chunk = p.m_chunk;
+  a.n_chunk = p.n_chunk;
+  a.m_tiles = ceil_div(p.m, p.m_chunk);
+  a.n_tiles = ceil_div(p.n, p.n_chunk);
+  constexpr size_t V = 16 / EB;
+  const size_t m_padded = a.m_tiles * a.m_chunk, n_padded = a.n_tiles * a.n_chunk;
+  if (p.batch == 0 || m_padded == 0 || n_padded == 0) return hipSuccess;
+  const bool vec_ok = (p.n_chunk % V == 0) && (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0) &&
+                      ((uintptr_t)p.out % 16 == 0) && p.batch <= 65535 &&
+                      ceil_div(m_padded, kRowsPerBlock) <= 65535;
+  if (vec_ok) {
+    a.n_vecs_padded = n_padded / V;
+    a.vecs_per_tile_row = p.n_chunk / V;
+    const dim3 grid((unsigned)ceil_div(a.n_vecs_padded, kVecsPerBlockRow),
+                    (unsigned)ceil_div(m_padded, kRowsPerBlock), (unsigned)p.batch);
+    if (p.interleaved) {
+      hipLaunchKernelGGL((transpose_vec<EB, true>), grid, dim3(256), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((transpose_vec<EB, false>), grid, dim3(256), 0, stream, a);
+    }
+  } else {
+    a.n_vecs_padded = 0;
+    a.vecs_per_tile_row = 0;
+    const size_t total = p.batch * m_padded * n_padded;
+    const size_t blocks = ceil_div(total, 256);
+    if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+    if (p.interleaved) {
+      hipLaunchKernelGGL((transpose_scalar<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                         a, p.batch);
+    } else {
+      hipLaunchKernelGGL((transpose_scalar<T, false>), dim3((unsigned)blocks), dim3(256), 0,
+                         stream, a, p.batch);
+    }
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_transpose(const TransposeParams &p, hipStream_t stream) {
+  switch (p.elem_bytes) {
+    case 1: return launch_width<1, unsigned char>(p, stream);
+    case 2: return launch_width<2, unsigned short>(p, stream);
+    case 4: return launch_width<4, unsigned>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace ccglib_amd

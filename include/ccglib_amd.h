@@ -1,0 +1,179 @@
+/*
+ * C ABI of the MI355X (gfx950) complex-GEMM library: plain pointers and sizes,
+ * opaque handles, integer status codes. These entry points are what the C++
+ * classes of the ccglib API bind to (include/ccglib/...): each section names the
+ * reference interface it stands in for, as file:line in the reference tree.
+ *
+ * Conventions
+ *  - Every function returns CCGLIB_OK (0) or a non-zero status; the text of the
+ *    last failure on the calling thread is returned by ccglib_last_error().
+ *  - `device` is a HIP device ordinal; `stream` is a hipStream_t passed as
+ *    void* (NULL = the default stream). All run functions only enqueue work on
+ *    that stream and return; they never synchronise, allocate or free, except
+ *    the *_run_host variants, which stage the host buffer through a
+ *    stream-ordered temporary.
+ *  - Pointers given to run functions are device pointers unless the name says
+ *    host. The library never owns caller buffers.
+ *  - Enum arguments are plain ints holding the values of the reference enums
+ *    (repeated below as CCGLIB_* constants).
+ *  - Objects are not thread-safe; use one per thread or serialise calls.
+ */
+#ifndef CCGLIB_AMD_H_
+#define CCGLIB_AMD_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CCGLIB_API __attribute__((visibility("default")))
+
+/* status codes */
+enum {
+  CCGLIB_OK = 0,
+  CCGLIB_ERROR_INVALID_ARGUMENT = 1, /* bad handle, null pointer, bad enum   */
+  CCGLIB_ERROR_UNSUPPORTED = 2,      /* valid request the library cannot do  */
+  CCGLIB_ERROR_RUNTIME = 3           /* a HIP call failed                    */
+};
+
+/* ValueType: include/ccglib/common/value_type.h:14-22 */
+enum {
+  CCGLIB_INT1 = 0,
+  CCGLIB_INT32 = 1,
+  CCGLIB_BFLOAT16 = 2,
+  CCGLIB_FLOAT8E4M3 = 3,
+  CCGLIB_FLOAT8E5M2 = 4,
+  CCGLIB_FLOAT16 = 5,
+  CCGLIB_FLOAT32 = 6
+};
+/* ComplexAxisLocation: include/ccglib/common/complex_order.h:12 */
+enum { CCGLIB_COMPLEX_PLANAR = 0, CCGLIB_COMPLEX_INTERLEAVED = 1 };
+/* Direction: include/ccglib/common/direction.h:6 */
+enum { CCGLIB_FORWARD = 0, CCGLIB_BACKWARD = 1 };
+/* MemOrder: include/ccglib/gemm/mem_order.h:6 */
+enum { CCGLIB_ROW_MAJOR = 0, CCGLIB_COL_MAJOR = 1 };
+/* Variant: include/ccglib/gemm/variant.h:6 */
+enum { CCGLIB_BASIC = 0, CCGLIB_OPT = 1 };
+
+typedef struct ccglib_gemm *ccglib_gemm_t;
+typedef struct ccglib_transpose *ccglib_transpose_t;
+typedef struct ccglib_packing *ccglib_packing_t;
+typedef struct ccglib_pipeline *ccglib_pipeline_t;
+
+/* Text of the last error raised on this thread ("" if none). */
+CCGLIB_API const char *ccglib_last_error(void);
+/* Library version string. */
+CCGLIB_API const char *ccglib_version(void);
+
+/* ------------------------------------------------------------------------
+ * Complex GEMM  C[b] = alpha * A[b] * B[b]^T + beta * C[b]
+ * Replaces ccglib::mma::GEMM: constructor include/ccglib/gemm/mma.h:42-49
+ * (src/mma/GEMM.cpp:243-254), Run :50 (src/mma/GEMM.cpp:263-268),
+ * GetDimensions :39-40 (src/mma/GEMM.cpp:270-275).
+ *
+ * Layouts (kernels/type_selector.h:224-241, kernels/gemm_kernel_float.cu:28-33):
+ *   basic: A [B][2][M][K], B [B][2][N][K] (K in 32-bit words for 1-bit input)
+ *   opt:   A [B][Mp/Mb][Kp/Kc][2][Mb][Kc], B likewise with Nb: the output of
+ *          the transpose below with the chunk sizes of get_dimensions
+ *   C:     planar [B][2][M][N] (row major) / [B][2][N][M] (column major);
+ *          interleaved [B][M][N][2] / [B][N][M][2] (opt variant only)
+ * Supported (type_in -> type_out): float16->float32|float16,
+ * bfloat16->float32|bfloat16, float8e4m3->float32, float8e5m2->float32,
+ * int1->int32. Accumulation is float32 (int32 for 1-bit input).
+ * a_order must be row major and b_order column major (as in the reference,
+ * where anything else fails to compile: kernels/gemm_kernel_float.cu:20-25);
+ * the error text keeps the token HIPRTC_ERROR_COMPILATION that the
+ * reference's callers match on (test/gemm/mma.cpp:598-627).
+ * 1-bit input: K must be a multiple of 32; alpha and beta are truncated to
+ * integers (src/reference/GEMM.cpp:202-205).
+ * C is read only when beta != 0.
+ * ---------------------------------------------------------------------- */
+CCGLIB_API int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M,
+                                  size_t N, size_t K, int device, void *stream,
+                                  int type_in, int type_out, int variant,
+                                  int c_complex_axis_location, int c_mem_order,
+                                  int a_mem_order, int b_mem_order,
+                                  float alpha_re, float alpha_im, float beta_re,
+                                  float beta_im);
+/* Argument order (a, b, c) as in GEMM::Run. */
+CCGLIB_API int ccglib_gemm_run(ccglib_gemm_t gemm, const void *d_a,
+                               const void *d_b, void *d_c);
+CCGLIB_API int ccglib_gemm_destroy(ccglib_gemm_t gemm);
+/* (m_per_block, n_per_block, k_chunk): the chunk sizes of the opt layout. */
+CCGLIB_API int ccglib_gemm_get_dimensions(int type_in, int type_out,
+                                          int variant, unsigned *m_per_block,
+                                          unsigned *n_per_block,
+                                          unsigned *k_chunk);
+
+/* ------------------------------------------------------------------------
+ * Transpose into the tiled layout of the opt GEMM.
+ * Replaces ccglib::transpose::Transpose: constructor
+ * include/ccglib/transpose/transpose.h:26-29
+ * (src/transpose/Transpose.cpp:131-141), Run(device) :31
+ * (src/transpose/Transpose.cpp:160-164), Run(host) :30 (a no-op in the
+ * reference, src/transpose/Transpose.cpp:147-154; here it does the work).
+ *   in  [B][2][M][N] (planar) or [B][M][N][2] (interleaved)
+ *   out [B][Mp/Mc][Np/Nc][2][Mc][Nc], zero where m >= M or n >= N
+ * nr_bits is 1, 8, 16 or 32; for 1 bit N and N_chunk count samples and must
+ * be multiples of 32 (whole 32-bit words move).
+ * ---------------------------------------------------------------------- */
+CCGLIB_API int ccglib_transpose_create(ccglib_transpose_t *transpose, size_t B,
+                                       size_t M, size_t N, size_t M_chunk,
+                                       size_t N_chunk, size_t nr_bits,
+                                       int device, void *stream,
+                                       int input_complex_axis_location);
+CCGLIB_API int ccglib_transpose_run(ccglib_transpose_t transpose,
+                                    const void *d_input, void *d_output);
+CCGLIB_API int ccglib_transpose_run_host(ccglib_transpose_t transpose,
+                                         const void *h_input, void *d_output);
+CCGLIB_API int ccglib_transpose_destroy(ccglib_transpose_t transpose);
+
+/* ------------------------------------------------------------------------
+ * Bit packing: N one-byte samples <-> N bits, LSB first in 32-bit words.
+ * Replaces ccglib::packing::Packing: constructor
+ * include/ccglib/packing/packing.h:35-38 (src/packing/Packing.cpp:136-141),
+ * Run(device) :40 (src/packing/Packing.cpp:162-166), Run(host) :39
+ * (src/packing/Packing.cpp:152-156).
+ * forward: byte != 0 -> bit 1; interleaved input (re,im pairs) is packed as all
+ * real bits followed by all imaginary bits (kernels/packing_kernel.cu:15-22).
+ * backward: bits -> bytes of 0/1, planar only (create fails otherwise, as
+ * src/packing/Packing.cpp:49-53). The packed buffer holds ceil(N/32) words.
+ * ---------------------------------------------------------------------- */
+CCGLIB_API int ccglib_packing_create(ccglib_packing_t *packing, size_t N,
+                                     int direction, int device, void *stream,
+                                     int input_complex_axis_location);
+CCGLIB_API int ccglib_packing_run(ccglib_packing_t packing,
+                                  const void *d_input, void *d_output);
+CCGLIB_API int ccglib_packing_run_host(ccglib_packing_t packing,
+                                       const void *h_input, void *d_output);
+CCGLIB_API int ccglib_packing_destroy(ccglib_packing_t packing);
+
+/* ------------------------------------------------------------------------
+ * Pipeline: [pack] -> [transpose] -> GEMM with scratch buffers owned by the
+ * object. Replaces ccglib::pipeline::Pipeline: constructor
+ * include/ccglib/pipeline/pipeline.h:44-53 (src/pipeline/Pipeline.cpp:145-160),
+ * Run(device) :54 (src/pipeline/Pipeline.cpp:183-188), Run(host) :41
+ * (src/pipeline/Pipeline.cpp:162-176).
+ * 1-bit input is one byte per sample and is packed first; the opt variant
+ * transposes A and B first. Argument order follows the reference constructor.
+ * run_host copies a, b (and c when beta != 0) to the device, runs, copies c
+ * back and synchronises the stream; sizes are those of the layouts above.
+ * ---------------------------------------------------------------------- */
+CCGLIB_API int ccglib_pipeline_create(
+    ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
+    int device, void *stream, int input_complex_axis_location,
+    int output_complex_axis_location, int a_mem_order, int b_mem_order,
+    int c_mem_order, int input_type, int output_type, int variant,
+    float alpha_re, float alpha_im, float beta_re, float beta_im);
+CCGLIB_API int ccglib_pipeline_run(ccglib_pipeline_t pipeline, const void *d_a,
+                                   const void *d_b, void *d_c);
+CCGLIB_API int ccglib_pipeline_run_host(ccglib_pipeline_t pipeline,
+                                        const void *h_a, const void *h_b,
+                                        void *h_c);
+CCGLIB_API int ccglib_pipeline_destroy(ccglib_pipeline_t pipeline);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CCGLIB_AMD_H_ */

@@ -1,0 +1,255 @@
+"""GPU parity tests of the complex GEMM against the CPU oracle, through the C ABI
+(ccglib_amd.GEMM / Transpose are thin ctypes bindings). Shapes and cases follow
+the reference's test/gemm/mma.cpp."""
+import numpy as np
+import pytest
+import torch
+
+import ccglib_amd as cc
+import oracle as orc
+from gpu_util import (ORC_TYPE, check_float, dequantize, device_zeros, quantize, stream,
+                      to_device, to_host, transpose_operand)
+
+pytestmark = pytest.mark.gpu
+
+VT = cc.ValueType
+PLANAR, INTERLEAVED = cc.ComplexAxisLocation.complex_planar, cc.ComplexAxisLocation.complex_interleaved
+ROW, COL = cc.MemOrder.row_major, cc.MemOrder.col_major
+OUT_NP = {VT.float32: np.float32, VT.float16: np.uint16, VT.bfloat16: np.uint16, VT.int32: np.int32}
+
+FLOAT_PAIRS = [(VT.float16, VT.float32), (VT.float16, VT.float16), (VT.bfloat16, VT.float32),
+               (VT.bfloat16, VT.bfloat16), (VT.float8e4m3, VT.float32), (VT.float8e5m2, VT.float32)]
+
+
+def run_gemm(qa, qb, B, M, N, K, tin, tout, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0,
+             c_in=None):
+    """Returns C as a numpy array in planar layout [B][2][rows][cols] of the
+    output storage type, whatever layout the GPU wrote."""
+    if variant == cc.Variant.opt:
+        d_a = transpose_operand(qa, B, M, K, tin)
+        d_b = transpose_operand(qb, B, N, K, tin)
+    else:
+        d_a, d_b = to_device(qa), to_device(qb)
+    out_np = OUT_NP[tout]
+    n_out = B * 2 * M * N
+    if c_in is not None:
+        c_dev_in = c_in
+        if c_axis == INTERLEAVED:
+            rows, cols = (M, N) if c_order == ROW else (N, M)
+            c_dev_in = np.ascontiguousarray(c_in.reshape(B, 2, rows, cols).transpose(0, 2, 3, 1))
+        d_c = to_device(c_dev_in.reshape(-1))
+    else:
+        # poison the output: every element must be written, none read
+        d_c = to_device(np.full(n_out, 0x7fc0 if out_np == np.uint16 else -1, dtype=out_np)
+                        if out_np != np.float32 else np.full(n_out, np.nan, dtype=np.float32))
+    gemm = cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(tin, tout), variant, c_axis, c_order,
+                   ROW, COL, alpha, beta)
+    gemm.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    c = to_host(d_c, out_np)
+    rows, cols = (M, N) if c_order == ROW else (N, M)
+    if c_axis == INTERLEAVED:
+        c = np.ascontiguousarray(c.reshape(B, rows, cols, 2).transpose(0, 3, 1, 2))
+    return c.reshape(B, 2, rows, cols)
+
+
+def reference_inputs(B, M, N, K, tin, signed, seed):
+    rng = np.random.default_rng(seed)
+    lo = -1.0 if signed else 0.0   # the reference's fixtures use [0, 1] (test/gemm/mma.cpp:144-217)
+    a = rng.uniform(lo, 1.0, (B, 2, M, K)).astype(np.float32)
+    b = rng.uniform(lo, 1.0, (B, 2, N, K)).astype(np.float32)
+    return quantize(a, tin).reshape(-1), quantize(b, tin).reshape(-1)
+
+
+def float_case(B, M, N, K, tin, tout, variant, c_axis, c_order, signed=True, alpha=1, beta=0, seed=0):
+    qa, qb = reference_inputs(B, M, N, K, tin, signed, seed)
+    c_in = None
+    if beta != 0:
+        rng = np.random.default_rng(seed + 1)
+        c32 = rng.uniform(0, 1, B * 2 * M * N).astype(np.float32)
+        c_in = c32 if tout == VT.float32 else quantize(c32, tout)
+    got = run_gemm(qa, qb, B, M, N, K, tin, tout, variant, c_axis, c_order, alpha, beta, c_in)
+    want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], int(c_order), alpha, beta, c_in)
+    gotf = dequantize(got, tout)
+    wantf = dequantize(want, tout)
+    want64 = orc.gemm_float64(qa, qb, M, N, K, ORC_TYPE[tin], int(c_order))
+    if alpha != 1 or beta != 0:
+        w = (want64[:, 0] + 1j * want64[:, 1]) * complex(alpha)
+        if beta != 0:
+            ci = dequantize(c_in, tout).reshape(want64.shape).astype(np.float64)
+            w = w + complex(beta) * (ci[:, 0] + 1j * ci[:, 1])
+        want64 = np.stack([w.real, w.imag], axis=1)
+    return check_float(gotf, wantf, want64, tin, tout)
+
+
+# ---- reference known answers, through the GPU --------------------------------------
+
+KAT_A = [1, 2, 3, 4, 5, 6, 6, 5, 4, 3, 2, 1]
+KAT_B = [1, 2, 3, 4, 4, 3, 2, 1]
+
+
+@pytest.mark.parametrize("tin", [VT.float16, VT.bfloat16])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_kat_float(tin, variant):
+    qa, qb = quantize(np.array(KAT_A), tin), quantize(np.array(KAT_B), tin)
+    c = run_gemm(qa, qb, 1, 3, 2, 2, tin, VT.float32, variant)
+    assert c.reshape(-1).tolist() == [-34, -6, -14, 14, 6, 34, 26, 42, 34, 34, 42, 26]
+    c = run_gemm(qa, qb, 1, 3, 2, 2, tin, VT.float32, variant, c_order=COL)
+    assert c.reshape(-1).tolist() == [-34, -14, 6, -6, 14, 34, 26, 34, 42, 42, 34, 26]
+
+
+def test_kat_alpha_beta_fp16():
+    seq = list(range(16)) + list(range(16, 0, -1))
+    q = quantize(np.array(seq), VT.float16)
+    c_in = np.array([0, 1, 2, 3, 4, 3, 2, 1], dtype=np.float32)
+    c = run_gemm(q, q.copy(), 1, 2, 2, 8, VT.float16, VT.float32, cc.Variant.basic,
+                 alpha=0.5 + 2.5j, beta=0.25 - 1.5j, c_in=c_in)
+    assert c.reshape(-1).tolist() == [-2110, -3039.25, -3040.5, -1409.75, -2571, 275.25, 273.5, 2607.75]
+
+
+def test_all_ones_closed_form():
+    # test/hip/mma.cpp:20-83: real part 0, imaginary part 2K
+    B, M, N, K = 3, 512, 512, 512
+    q = quantize(np.ones(B * 2 * M * K), VT.float16)
+    c = run_gemm(q, q.copy(), B, M, N, K, VT.float16, VT.float32, cc.Variant.basic)
+    assert np.all(c[:, 0] == 0) and np.all(c[:, 1] == 2 * K)
+
+
+# ---- the reference's fixture: B = 16, aligned and ragged shapes ------------------------
+
+SHAPES = [(128, 256, 64), (100, 60, 40)]   # test/gemm/mma.cpp:402-408
+
+
+@pytest.mark.parametrize("tin,tout", FLOAT_PAIRS)
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_basic(tin, tout, M, N, K, c_order):
+    float_case(16, M, N, K, tin, tout, cc.Variant.basic, PLANAR, c_order, signed=False)
+    float_case(16, M, N, K, tin, tout, cc.Variant.basic, PLANAR, c_order, signed=True, seed=3)
+
+
+@pytest.mark.parametrize("tin,tout", FLOAT_PAIRS)
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("c_order", [ROW, COL])
+@pytest.mark.parametrize("c_axis", [PLANAR, INTERLEAVED])
+def test_opt(tin, tout, M, N, K, c_order, c_axis):
+    float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=False)
+    float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=True, seed=5)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000),
+                                   (257, 129, 72), (130, 2, 2049)])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_odd_shapes_fp16(M, N, K, variant):
+    float_case(2, M, N, K, VT.float16, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
+
+
+@pytest.mark.parametrize("tin", [VT.float8e4m3, VT.float8e5m2])
+@pytest.mark.parametrize("K", [1, 63, 64, 65, 128, 192, 200])
+def test_fp8_k_tails(tin, K):
+    # an MFMA consumes two 64-value K tiles; odd tile counts and ragged tails
+    float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=K)
+    float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.opt, PLANAR, COL, seed=K + 1)
+
+
+@pytest.mark.parametrize("m", [255, 256])     # test/gemm/mma.cpp:645-711
+@pytest.mark.parametrize("variant,c_axis", [(cc.Variant.basic, PLANAR), (cc.Variant.opt, PLANAR),
+                                            (cc.Variant.opt, INTERLEAVED)])
+def test_alpha_beta_fp16(m, variant, c_axis):
+    float_case(16, m, 128, 256, VT.float16, VT.float32, variant, c_axis, ROW, signed=False,
+               alpha=0.3 + 1.6j, beta=0.8 - 1.1j)
+
+
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float16), (VT.bfloat16, VT.bfloat16)])
+def test_alpha_beta_narrow_output(tin, tout):
+    float_case(4, 100, 60, 40, tin, tout, cc.Variant.opt, PLANAR, COL, alpha=-0.5 + 0.25j,
+               beta=1.5 + 0.5j)
+
+
+def test_beta_zero_ignores_nan_in_c():
+    # run_gemm poisons C with NaN whenever beta == 0: every float case above covers
+    # it; this one states the property on its own
+    qa, qb = reference_inputs(1, 8, 8, 8, VT.float16, True, 0)
+    c = run_gemm(qa, qb, 1, 8, 8, 8, VT.float16, VT.float32, cc.Variant.basic)
+    assert np.isfinite(c).all()
+
+
+def test_config1_reference_cpu_case():
+    # batch 1, 256^3, fp16 in, fp32 out, U[-1, 1]
+    for variant in (cc.Variant.basic, cc.Variant.opt):
+        float_case(1, 256, 256, 256, VT.float16, VT.float32, variant, PLANAR, ROW, seed=1)
+
+
+def test_batches_are_independent():
+    qa, qb = reference_inputs(4, 96, 80, 64, VT.bfloat16, True, 9)
+    full = run_gemm(qa, qb, 4, 96, 80, 64, VT.bfloat16, VT.float32, cc.Variant.opt)
+    a4, b4 = qa.reshape(4, -1), qb.reshape(4, -1)
+    for i in range(4):
+        one = run_gemm(a4[i].copy(), b4[i].copy(), 1, 96, 80, 64, VT.bfloat16, VT.float32,
+                       cc.Variant.opt)
+        assert np.array_equal(one[0], full[i])
+
+
+# ---- 1-bit ------------------------------------------------------------------------------
+
+def int1_case(B, M, N, K, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0, seed=0):
+    rng = np.random.default_rng(seed)
+    kw = (K + 31) // 32
+    mask = np.full(kw, 0xFFFFFFFF, dtype=np.uint32)
+    if K % 32:
+        mask[-1] = (1 << (K % 32)) - 1
+    a = (rng.integers(0, 2 ** 32, (B, 2, M, kw), dtype=np.uint32) & mask).reshape(-1)
+    b = (rng.integers(0, 2 ** 32, (B, 2, N, kw), dtype=np.uint32) & mask).reshape(-1)
+    c_in = rng.integers(-2 ** 30, 2 ** 30, B * 2 * M * N).astype(np.int32)
+    d_a = transpose_operand(a, B, M, K, VT.int1) if variant == cc.Variant.opt else to_device(a)
+    d_b = transpose_operand(b, B, N, K, VT.int1) if variant == cc.Variant.opt else to_device(b)
+    rows, cols = (M, N) if c_order == ROW else (N, M)
+    c_dev = c_in.reshape(B, 2, rows, cols)
+    if c_axis == INTERLEAVED:
+        c_dev = c_dev.transpose(0, 2, 3, 1)
+    d_c = to_device(np.ascontiguousarray(c_dev).reshape(-1))
+    cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.int1, VT.int32), variant, c_axis, c_order,
+            ROW, COL, alpha, beta).Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, np.int32)
+    if c_axis == INTERLEAVED:
+        got = got.reshape(B, rows, cols, 2).transpose(0, 3, 1, 2)
+    want = orc.gemm(a, b, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, c_in)
+    assert np.array_equal(got.reshape(want.shape), want)
+
+
+def test_kat_int1():
+    a = np.array([4007499276, 2587246816, 2368114480, 2180517764], dtype=np.uint32)
+    b = np.array([3172811225, 4156143586, 144478092, 808068269], dtype=np.uint32)
+    for c_in, alpha, beta, want in [
+            (np.zeros(8, np.int32), 1, 0, [-8, 8, -10, -6, 8, -12, -6, 6]),
+            (np.arange(1, 9, dtype=np.int32), 2 + 3j, -1 + 2j, [-51, 38, -19, -50, -11, -2, -43, -6])]:
+        d_a, d_b, d_c = to_device(a), to_device(b), to_device(c_in)
+        cc.GEMM(1, 2, 2, 32, 0, stream(), cc.Precision(VT.int1, VT.int32), cc.Variant.basic, PLANAR,
+                ROW, ROW, COL, alpha, beta).Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+        torch.cuda.synchronize()
+        assert to_host(d_c, np.int32).tolist() == want
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+@pytest.mark.parametrize("c_order", [ROW, COL])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 256), (128, 128, 512), (100, 60, 1024), (130, 257, 96),
+                                   (256, 128, 4096)])
+def test_int1(variant, c_order, M, N, K):
+    int1_case(16 if M == 64 else 3, M, N, K, variant, PLANAR, c_order, seed=M)
+
+
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_int1_interleaved_output(c_order):
+    int1_case(2, 100, 60, 512, cc.Variant.opt, INTERLEAVED, c_order)
+
+
+@pytest.mark.parametrize("K", [45, 100])
+def test_int1_k_not_multiple_of_32(K):
+    int1_case(2, 20, 30, K, cc.Variant.basic, seed=K)
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_int1_alpha_beta(variant):
+    # test/gemm/mma.cpp:713-775
+    int1_case(16, 256, 128, 256, variant, alpha=2 - 3j, beta=3 - 2j)

@@ -1,0 +1,80 @@
+"""GPU parity tests of the pipeline wrapper (pack -> transpose -> GEMM) against the
+CPU oracle; cases follow the reference's test/pipeline/pipeline.cpp."""
+import numpy as np
+import pytest
+import torch
+
+import ccglib_amd as cc
+import oracle as orc
+from gpu_util import ORC_TYPE, check_float, quantize, stream, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+VT = cc.ValueType
+PLANAR, INTERLEAVED = cc.ComplexAxisLocation.complex_planar, cc.ComplexAxisLocation.complex_interleaved
+ROW, COL = cc.MemOrder.row_major, cc.MemOrder.col_major
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.opt, cc.Variant.basic])
+@pytest.mark.parametrize("host", [False, True])
+def test_pipeline_float16(variant, host):
+    # test/pipeline/pipeline.cpp:17-86
+    B, M, N, K = 2, 300, 200, 100
+    alpha, beta = 1.5 - 1.5j, 0.5 - 0.5j
+    rng = np.random.default_rng(0)
+    qa = quantize(rng.uniform(-10, 10, B * 2 * M * K), VT.float16)
+    qb = quantize(rng.uniform(-10, 10, B * 2 * N * K), VT.float16)
+    c_in = rng.uniform(-10, 10, B * 2 * M * N).astype(np.float32)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, VT.float16, VT.float32,
+                    variant, alpha, beta)
+    if host:
+        got = c_in.copy()
+        p.RunHost(qa.ctypes.data, qb.ctypes.data, got.ctypes.data)
+    else:
+        d_a, d_b, d_c = to_device(qa), to_device(qb), to_device(c_in)
+        p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+        torch.cuda.synchronize()
+        got = to_host(d_c, np.float32)
+    want = orc.gemm(qa, qb, M, N, K, orc.FLOAT16, orc.FLOAT32, orc.ROW_MAJOR, alpha, beta, c_in)
+    w64 = orc.gemm_float64(qa, qb, M, N, K, orc.FLOAT16)
+    w = (w64[:, 0] + 1j * w64[:, 1]) * alpha + beta * (c_in.reshape(B, 2, M, N)[:, 0].astype(np.float64)
+                                                       + 1j * c_in.reshape(B, 2, M, N)[:, 1])
+    check_float(got.reshape(want.shape), want, np.stack([w.real, w.imag], 1), VT.float16, VT.float32)
+
+
+def test_pipeline_interleaved_in_and_out():
+    B, M, N, K = 3, 130, 70, 96
+    rng = np.random.default_rng(1)
+    a = rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32)
+    qa, qb = quantize(a, VT.bfloat16), quantize(b, VT.bfloat16)
+    qa_il = np.ascontiguousarray(qa.transpose(0, 2, 3, 1))
+    qb_il = np.ascontiguousarray(qb.transpose(0, 2, 3, 1))
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, INTERLEAVED, ROW, COL, COL, VT.bfloat16,
+                    VT.float32, cc.Variant.opt)
+    d_a, d_b = to_device(qa_il.reshape(-1)), to_device(qb_il.reshape(-1))
+    d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, np.float32).reshape(B, N, M, 2).transpose(0, 3, 1, 2)
+    want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, orc.BFLOAT16, orc.FLOAT32, orc.COL_MAJOR)
+    w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, orc.BFLOAT16, orc.COL_MAJOR)
+    check_float(got, want, w64, VT.bfloat16, VT.float32)
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.opt, cc.Variant.basic])
+def test_pipeline_int1(variant):
+    # test/pipeline/pipeline.cpp:88-187: one byte per sample in, packed inside
+    B, M, N, K = 2, 512, 512, 512
+    alpha, beta = 2 + 3j, 1 - 3j
+    rng = np.random.default_rng(2)
+    a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8)
+    c_in = rng.integers(-2 ** 31, 2 ** 31, B * 2 * M * N).astype(np.int32)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                    variant, alpha, beta)
+    d_a, d_b, d_c = to_device(a_bits), to_device(b_bits), to_device(c_in)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    want = orc.gemm(orc.pack_bits(a_bits), orc.pack_bits(b_bits), M, N, K, orc.INT1, orc.INT32,
+                    orc.ROW_MAJOR, alpha, beta, c_in)
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
