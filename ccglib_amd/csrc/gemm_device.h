@@ -93,6 +93,7 @@ struct KernelArgs {
   size_t x_batch_bytes, y_batch_bytes;
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta, c_interleaved;
+  int c_vector_ok;  // C base is 16-byte aligned: wide stores allowed
 };
 
 // Maps the hardware workgroup id to a logical tile id such that the ids that
@@ -164,6 +165,7 @@ inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
   a.have_alpha = p.have_alpha;
   a.have_beta = p.have_beta;
   a.c_interleaved = p.c_interleaved;
+  a.c_vector_ok = ((uintptr_t)p.c % 16 == 0);
   return a;
 }
 

@@ -232,7 +232,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const bool have_alpha = args.have_alpha, have_beta = args.have_beta;
   const float ar = args.alpha_re, ai = args.alpha_im, br = args.beta_re, bi = args.beta_im;
   Tout *cbase = reinterpret_cast<Tout *>(args.c) + (size_t)b * 2 * nx * ny;
-  const bool vec_ok = (nx % 4 == 0);
+  const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
     const unsigned y = block_y * BY + wy * WY + j * 16 + (lane & 15);
