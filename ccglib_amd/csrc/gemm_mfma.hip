@@ -7,9 +7,11 @@
 // products per complex product (gemm_kernel_float.cu:293-303); everything
 // else is laid out for 64-wide wavefronts:
 //
-//  * One block owns a BX x BY patch of C and walks K in stages of KT tiles of
-//    64 bytes. Operand tiles are staged global -> registers -> LDS one stage
-//    ahead of the math (two LDS stages, one barrier per stage).
+//  * One block owns a BX x BY patch of C and walks K in tiles of 64 bytes.
+//    For the tiled (opt) layout the tiles go global -> LDS directly
+//    (global_load_lds_dwordx4) through a ring of LDS slots, two iterations
+//    ahead of the math; the planar (basic) layouts are staged through
+//    registers, which is where their bounds checks and zero fill happen.
 //  * LDS rows are 64 bytes; the 16-byte chunk index is XORed with
 //    (row >> 1) & 3, which makes both the linear 16-byte writes and the
 //    16-row fragment reads free of bank conflicts on this LDS.
@@ -88,146 +90,54 @@ template <> struct OutType<kFloat32> { using type = float; };
 template <> struct OutType<kFloat16> { using type = _Float16; };
 template <> struct OutType<kBfloat16> { using type = __bf16; };
 
-template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WAVES_PER_EU>
-__global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma(
-    const KernelArgs args) {
-  using Tout = typename OutType<TOUT>::type;
-  constexpr int NWX = BX / WX, NWY = BY / WY;
-  constexpr int NTHREADS = 64 * NWX * NWY;
-  constexpr int TX = WX / 16, TY = WY / 16;
+// One K tile (or two for fp8) of math for a wave: reads its X and Y fragments
+// from the LDS slot(s) and issues the four real products of the complex MAC.
+// slot[u] points at the K tile u of this MFMA step: [X re][X im][Y re][Y im].
+template <int DT, int BX, int BY, int TX, int TY>
+__device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<DT>::kTilesPerMfma],
+                                         int x_frag_off, int y_frag_off,
+                                         float4_t (&acc_re)[TY][TX], float4_t (&acc_im)[TY][TX]) {
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
-  static_assert(KT % KPM == 0, "stage must hold whole MFMAs");
-  constexpr int X_KTILE_BYTES = 2 * BX * kTileRowBytes;
-  constexpr int Y_KTILE_BYTES = 2 * BY * kTileRowBytes;
-  constexpr int KTILE_BYTES = X_KTILE_BYTES + Y_KTILE_BYTES;
-  constexpr int STAGE_BYTES = KT * KTILE_BYTES;
-  constexpr int X_CHUNKS = KT * 2 * BX * 4;
-  constexpr int Y_CHUNKS = KT * 2 * BY * 4;
-  static_assert(X_CHUNKS % NTHREADS == 0 && Y_CHUNKS % NTHREADS == 0, "chunks per thread");
-  constexpr int CX = X_CHUNKS / NTHREADS, CY = Y_CHUNKS / NTHREADS;
-
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wx = wave % NWX, wy = wave / NWX;
-
-  // ---- which tile of C -------------------------------------------------
-  const TileCoord tc = tile_coord(args, blockIdx.x);
-  const unsigned b = tc.b, block_x = tc.block_x, block_y = tc.block_y;
-
-  OperandView xv{args.x + (size_t)b * args.x_batch_bytes, args.nx, args.x_tiles, block_x * BX};
-  OperandView yv{args.y + (size_t)b * args.y_batch_bytes, args.ny, args.y_tiles, block_y * BY};
-  const unsigned k_tiles = args.k_tiles;
-  const unsigned k_bytes = args.k_bytes;
-
-  // ---- staging registers and their LDS destinations --------------------
-  int4_t xs[CX], ys[CY];
-  auto fetch = [&](unsigned kt0) {
+  Fragment<DT> xr[TX], xi[TX];
 #pragma unroll
-    for (int i = 0; i < CX; ++i) {
-      const int gidx = tid + i * NTHREADS;
-      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
-      xs[i] = load_chunk<DtypeTraits<DT>::kElemBytes, LOADER>(
-          xv, kt0 + kk, k_tiles, k_bytes, rem / (BX * 4), (rem / 4) % BX, rem % 4);
-    }
+  for (int i = 0; i < TX; ++i) {
 #pragma unroll
-    for (int i = 0; i < CY; ++i) {
-      const int gidx = tid + i * NTHREADS;
-      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
-      ys[i] = load_chunk<DtypeTraits<DT>::kElemBytes, LOADER>(
-          yv, kt0 + kk, k_tiles, k_bytes, rem / (BY * 4), (rem / 4) % BY, rem % 4);
+    for (int u = 0; u < KPM; ++u) {
+      const char *p = slot[u] + x_frag_off + i * 16 * kTileRowBytes;
+      xr[i].v[u] = *reinterpret_cast<const int4_t *>(p);
+      xi[i].v[u] = *reinterpret_cast<const int4_t *>(p + BX * kTileRowBytes);
     }
-  };
-  auto stash = [&](int stage) {
-    char *s = lds + stage * STAGE_BYTES;
-#pragma unroll
-    for (int i = 0; i < CX; ++i) {
-      const int gidx = tid + i * NTHREADS;
-      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
-      const int plane = rem / (BX * 4), row = (rem / 4) % BX, c = rem % 4;
-      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + plane * BX * kTileRowBytes +
-                                  swizzled_row_offset(row, c)) = xs[i];
-    }
-#pragma unroll
-    for (int i = 0; i < CY; ++i) {
-      const int gidx = tid + i * NTHREADS;
-      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
-      const int plane = rem / (BY * 4), row = (rem / 4) % BY, c = rem % 4;
-      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + X_KTILE_BYTES +
-                                  plane * BY * kTileRowBytes + swizzled_row_offset(row, c)) =
-          ys[i];
-    }
-  };
-
-  // ---- accumulators ------------------------------------------------------
-  float4_t acc_re[TY][TX], acc_im[TY][TX];
+  }
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
+    Fragment<DT> yr, yi;
 #pragma unroll
-    for (int i = 0; i < TX; ++i) {
-      acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
-      acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < KPM; ++u) {
+      const char *p = slot[u] + y_frag_off + j * 16 * kTileRowBytes;
+      yr.v[u] = *reinterpret_cast<const int4_t *>(p);
+      yi.v[u] = *reinterpret_cast<const int4_t *>(p + BY * kTileRowBytes);
     }
+    const Fragment<DT> yin = negate<DT>(yi);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xr[i], yr, acc_re[j][i]);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xr[i], yi, acc_im[j][i]);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
   }
+}
 
-  const int lane_off = swizzled_row_offset(lane & 15, lane >> 4);
-  const int x_frag_base = (wx * WX) * kTileRowBytes + lane_off;
-  const int y_frag_base = X_KTILE_BYTES + (wy * WY) * kTileRowBytes + lane_off;
-
-  auto compute = [&](int stage) {
-    const char *s = lds + stage * STAGE_BYTES;
-#pragma unroll
-    for (int kk = 0; kk < KT; kk += KPM) {
-      Fragment<DT> xr[TX], xi[TX];
-#pragma unroll
-      for (int i = 0; i < TX; ++i) {
-#pragma unroll
-        for (int u = 0; u < KPM; ++u) {
-          const char *p = s + (kk + u) * KTILE_BYTES + x_frag_base + i * 16 * kTileRowBytes;
-          xr[i].v[u] = *reinterpret_cast<const int4_t *>(p);
-          xi[i].v[u] = *reinterpret_cast<const int4_t *>(p + BX * kTileRowBytes);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < TY; ++j) {
-        Fragment<DT> yr, yi;
-#pragma unroll
-        for (int u = 0; u < KPM; ++u) {
-          const char *p = s + (kk + u) * KTILE_BYTES + y_frag_base + j * 16 * kTileRowBytes;
-          yr.v[u] = *reinterpret_cast<const int4_t *>(p);
-          yi.v[u] = *reinterpret_cast<const int4_t *>(p + BY * kTileRowBytes);
-        }
-        const Fragment<DT> yin = negate<DT>(yi);
-#pragma unroll
-        for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xr[i], yr, acc_re[j][i]);
-#pragma unroll
-        for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xr[i], yi, acc_im[j][i]);
-#pragma unroll
-        for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
-#pragma unroll
-        for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
-      }
-    }
-  };
-
-  // ---- main loop ---------------------------------------------------------
-  const unsigned stages = (k_tiles + KT - 1) / KT;
-  fetch(0);
-  stash(0);
-  if (stages > 1) fetch(KT);
-  __syncthreads();
-  for (unsigned s = 0; s < stages; ++s) {
-    const int cur = s & 1;
-    if (s + 1 < stages) stash(cur ^ 1);
-    if (s + 2 < stages) fetch((s + 2) * KT);
-    compute(cur);
-    __syncthreads();
-  }
-
-  // ---- epilogue: alpha * acc + beta * C, store ---------------------------
-  // lane holds, per 16x16 tile, x = x0 + (lane/16)*4 + 0..3 at y = y0 + lane%16
+// Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
+// store. The lane holds, per 16x16 tile, x = x0 + (lane/16)*4 + 0..3 at
+// y = y0 + lane%16, i.e. four consecutive elements of the contiguous C axis.
+template <int TOUT, int TX, int TY>
+__device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned b, unsigned x_wave,
+                                                unsigned y_wave, int lane,
+                                                float4_t (&acc_re)[TY][TX],
+                                                float4_t (&acc_im)[TY][TX]) {
+  using Tout = typename OutType<TOUT>::type;
   const unsigned nx = args.nx, ny = args.ny;
   const bool have_alpha = args.have_alpha, have_beta = args.have_beta;
   const float ar = args.alpha_re, ai = args.alpha_im, br = args.beta_re, bi = args.beta_im;
@@ -235,10 +145,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
-    const unsigned y = block_y * BY + wy * WY + j * 16 + (lane & 15);
+    const unsigned y = y_wave + j * 16 + (lane & 15);
 #pragma unroll
     for (int i = 0; i < TX; ++i) {
-      const unsigned x = block_x * BX + wx * WX + i * 16 + (lane >> 4) * 4;
+      const unsigned x = x_wave + i * 16 + (lane >> 4) * 4;
       if (y >= ny || x >= nx) continue;
       float re[4], im[4];
 #pragma unroll
@@ -319,6 +229,268 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   }
 }
 
+// ---------------------------------------------------------------------------
+// Register-staged kernel: global -> registers -> LDS, two LDS stages. Used for
+// the planar (basic) layouts, whose loads need bounds checks and zero fill.
+// ---------------------------------------------------------------------------
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WAVES_PER_EU>
+__global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma(
+    const KernelArgs args) {
+  constexpr int NWX = BX / WX, NWY = BY / WY;
+  constexpr int NTHREADS = 64 * NWX * NWY;
+  constexpr int TX = WX / 16, TY = WY / 16;
+  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr int EB = DtypeTraits<DT>::kElemBytes;
+  static_assert(KT % KPM == 0, "stage must hold whole MFMAs");
+  constexpr int X_KTILE_BYTES = 2 * BX * kTileRowBytes;
+  constexpr int Y_KTILE_BYTES = 2 * BY * kTileRowBytes;
+  constexpr int KTILE_BYTES = X_KTILE_BYTES + Y_KTILE_BYTES;
+  constexpr int STAGE_BYTES = KT * KTILE_BYTES;
+  constexpr int X_CHUNKS = KT * 2 * BX * 4;
+  constexpr int Y_CHUNKS = KT * 2 * BY * 4;
+  static_assert(X_CHUNKS % NTHREADS == 0 && Y_CHUNKS % NTHREADS == 0, "chunks per thread");
+  constexpr int CX = X_CHUNKS / NTHREADS, CY = Y_CHUNKS / NTHREADS;
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wx = wave % NWX, wy = wave / NWX;
+
+  const TileCoord tc = tile_coord(args, blockIdx.x);
+  const unsigned b = tc.b, block_x = tc.block_x, block_y = tc.block_y;
+
+  OperandView xv{args.x + (size_t)b * args.x_batch_bytes, args.nx, args.x_tiles, block_x * BX};
+  OperandView yv{args.y + (size_t)b * args.y_batch_bytes, args.ny, args.y_tiles, block_y * BY};
+  const unsigned k_tiles = args.k_tiles;
+  const unsigned k_bytes = args.k_bytes;
+
+  int4_t xs[CX], ys[CY];
+  auto fetch = [&](unsigned kt0) {
+#pragma unroll
+    for (int i = 0; i < CX; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
+      xs[i] = load_chunk<EB, LOADER>(xv, kt0 + kk, k_tiles, k_bytes, rem / (BX * 4),
+                                     (rem / 4) % BX, rem % 4);
+    }
+#pragma unroll
+    for (int i = 0; i < CY; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
+      ys[i] = load_chunk<EB, LOADER>(yv, kt0 + kk, k_tiles, k_bytes, rem / (BY * 4),
+                                     (rem / 4) % BY, rem % 4);
+    }
+  };
+  auto stash = [&](int stage) {
+    char *s = lds + stage * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < CX; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BX * 4), rem = gidx % (2 * BX * 4);
+      const int plane = rem / (BX * 4), row = (rem / 4) % BX, c = rem % 4;
+      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + plane * BX * kTileRowBytes +
+                                  swizzled_row_offset(row, c)) = xs[i];
+    }
+#pragma unroll
+    for (int i = 0; i < CY; ++i) {
+      const int gidx = tid + i * NTHREADS;
+      const int kk = gidx / (2 * BY * 4), rem = gidx % (2 * BY * 4);
+      const int plane = rem / (BY * 4), row = (rem / 4) % BY, c = rem % 4;
+      *reinterpret_cast<int4_t *>(s + kk * KTILE_BYTES + X_KTILE_BYTES +
+                                  plane * BY * kTileRowBytes + swizzled_row_offset(row, c)) =
+          ys[i];
+    }
+  };
+
+  float4_t acc_re[TY][TX], acc_im[TY][TX];
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+#pragma unroll
+    for (int i = 0; i < TX; ++i) {
+      acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  const int lane_off = swizzled_row_offset(lane & 15, lane >> 4);
+  const int x_frag_off = (wx * WX) * kTileRowBytes + lane_off;
+  const int y_frag_off = X_KTILE_BYTES + (wy * WY) * kTileRowBytes + lane_off;
+
+  auto compute = [&](int stage) {
+    const char *s = lds + stage * STAGE_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < KT; kk += KPM) {
+      const char *slot[KPM];
+#pragma unroll
+      for (int u = 0; u < KPM; ++u) slot[u] = s + (kk + u) * KTILE_BYTES;
+      mma_step<DT, BX, BY, TX, TY>(slot, x_frag_off, y_frag_off, acc_re, acc_im);
+    }
+  };
+
+  const unsigned stages = (k_tiles + KT - 1) / KT;
+  fetch(0);
+  stash(0);
+  if (stages > 1) fetch(KT);
+  __syncthreads();
+  for (unsigned s = 0; s < stages; ++s) {
+    const int cur = s & 1;
+    if (s + 1 < stages) stash(cur ^ 1);
+    if (s + 2 < stages) fetch((s + 2) * KT);
+    compute(cur);
+    __syncthreads();
+  }
+
+  store_wave_tile<TOUT, TX, TY>(args, b, block_x * BX + wx * WX, block_y * BY + wy * WY, lane,
+                                acc_re, acc_im);
+}
+
+// ---------------------------------------------------------------------------
+// Direct-to-LDS kernel for the tiled (opt) layout. Operand tiles are contiguous
+// 16 KiB blocks, so the copy into LDS needs no registers: every wave issues
+// global_load_lds_dwordx4, each of which moves 16 rows x 64 bytes (1 KiB)
+// straight into LDS. The hardware writes lane L's 16 bytes at LDS offset
+// base + 16 L; the XOR swizzle of the LDS layout is obtained by letting lane L
+// fetch the chunk that belongs there (a permutation inside each 64-byte row,
+// so the global access stays fully coalesced).
+//
+// LDS is a ring of SLOTS K tiles. Iteration i waits for its own tile(s) with
+// s_waitcnt vmcnt(n) - n being the loads issued for later iterations - then
+// passes one barrier, issues the loads LEAD iterations ahead into the slot(s)
+// that the previous iteration just released, and does the math. Loads past
+// the end of K are pointed at a zero tile so that the count of outstanding
+// loads is the same in every iteration.
+// ---------------------------------------------------------------------------
+__device__ __attribute__((aligned(256))) char g_zero_tile[kTileBytes];
+
+template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_offset,
+                                               unsigned lds_address) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_address), "v"(lane_offset), "s"(base)
+      : "memory");
+}
+
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU>
+__global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma_dtl(
+    const KernelArgs args) {
+  constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
+  constexpr int TX = WX / 16, TY = WY / 16;
+  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr int X_BYTES = 2 * BX * kTileRowBytes;
+  constexpr int SLOT_BYTES = X_BYTES + 2 * BY * kTileRowBytes;
+  constexpr int ROW_BLOCKS = SLOT_BYTES / 1024;     // 16 rows x 64 bytes each
+  constexpr int X_ROW_BLOCKS = X_BYTES / 1024;
+  static_assert(ROW_BLOCKS % NW == 0, "row blocks must divide evenly over the waves");
+  constexpr int LPW = ROW_BLOCKS / NW;              // loads per wave per K tile
+  static_assert(SLOTS % KPM == 0 && SLOTS / KPM >= 2, "ring must hold at least two steps");
+  constexpr int LEAD = SLOTS / KPM - 1;             // iterations of prefetch distance
+  static_assert((LEAD - 1) * KPM * LPW < 64, "vmcnt range");
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wx = wave % NWX, wy = wave / NWX;
+
+  const TileCoord tc = tile_coord(args, blockIdx.x);
+  const unsigned b = tc.b, block_x = tc.block_x, block_y = tc.block_y;
+  const unsigned k_tiles = args.k_tiles;
+
+  // ---- this wave's share of the copy: LPW row blocks of every K tile ------
+  // row block q of a slot: X re, X im, Y re, Y im, 16 rows each
+  const char *src[LPW];        // wave-uniform: start of the operand tile row (K tile 0)
+  unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
+  unsigned lane_off[LPW];      // per lane: where this lane's 16 bytes come from
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
+  {
+    const int r = lane >> 2;                                  // row inside the row block
+    const int c = (lane & 3) ^ ((r >> 1) & 3);                // chunk that belongs at lane*16
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int q = i * NW + wave;
+      const bool is_x = q < X_ROW_BLOCKS;
+      const int qq = is_x ? q : q - X_ROW_BLOCKS;
+      const int rows = is_x ? BX : BY;
+      const int plane = qq / (rows / 16), rb = qq % (rows / 16);
+      const unsigned row0 = (is_x ? block_x * BX : block_y * BY) + rb * 16;
+      const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
+      unsigned tile = row0 / kTileRows;
+      tile = tile < tiles ? tile : tiles - 1;   // rows past the end: any valid data, never stored
+      const char *op = is_x ? args.x + (size_t)b * args.x_batch_bytes
+                            : args.y + (size_t)b * args.y_batch_bytes;
+      src[i] = op + (size_t)tile * k_tiles * kTileBytes;
+      lane_off[i] = plane * kTilePlaneBytes + ((row0 % kTileRows) + r) * kTileRowBytes + c * 16;
+      lds_dst[i] = lds_base + q * 1024;
+    }
+  }
+  auto issue = [&](unsigned kt, int slot) {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const char *base = kt < k_tiles ? src[i] + (size_t)kt * kTileBytes : g_zero_tile;
+      load_1k_to_lds(base, lane_off[i], lds_dst[i] + slot * SLOT_BYTES);
+    }
+  };
+
+  float4_t acc_re[TY][TX], acc_im[TY][TX];
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+#pragma unroll
+    for (int i = 0; i < TX; ++i) {
+      acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
+  const int x_frag_off = (wx * WX) * kTileRowBytes + frag_lane_off;
+  const int y_frag_off = X_BYTES + (wy * WY) * kTileRowBytes + frag_lane_off;
+
+  // ---- pipeline ----------------------------------------------------------
+  const unsigned iters = (k_tiles + KPM - 1) / KPM;
+#pragma unroll
+  for (int t = 0; t < LEAD * KPM; ++t) issue(t, t);
+  unsigned slot = 0;                       // first slot of the current iteration
+  for (unsigned it = 0; it < iters; ++it) {
+    wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
+    // the slots of iteration it-1 are free now: refill them for iteration it+LEAD
+    unsigned refill = slot + LEAD * KPM;
+    refill = refill >= SLOTS ? refill - SLOTS : refill;
+#pragma unroll
+    for (int u = 0; u < KPM; ++u) issue((it + LEAD) * KPM + u, refill + u);
+    const char *tile[KPM];
+#pragma unroll
+    for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
+    mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
+    slot += KPM;
+    slot = slot >= SLOTS ? slot - SLOTS : slot;
+  }
+  // nothing may still be writing into LDS when the block gives it back
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  store_wave_tile<TOUT, TX, TY>(args, b, block_x * BX + wx * WX, block_y * BY + wy * WY, lane,
+                                acc_re, acc_im);
+}
+
+inline hipError_t check_grid(size_t total) {
+  return total > 0x7fffffffu ? hipErrorInvalidValue : hipSuccess;
+}
+
+// LDS beyond 64 KiB has to be requested once per kernel.
+template <typename Kernel> hipError_t allow_lds(Kernel kernel, int bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WPE>
 hipError_t launch_config(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
@@ -326,37 +498,51 @@ hipError_t launch_config(const GemmParams &p, hipStream_t stream) {
   const KernelArgs a = make_kernel_args(p, BX, BY);
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
-  if (total > 0x7fffffffu) return hipErrorInvalidValue;
+  if (hipError_t e = check_grid(total)) return e;
   auto kernel = complex_gemm_mfma<DT, TOUT, BX, BY, WX, WY, KT, LOADER, WPE>;
-  if (LDS_BYTES > 64 * 1024) {
-    static bool raised = false;  // per instantiation
-    if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-      if (e != hipSuccess) return e;
-      raised = true;
-    }
-  }
+  static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
+  if (lds_ok != hipSuccess) return lds_ok;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(NTHREADS), LDS_BYTES, stream, a);
+  return hipGetLastError();
+}
+
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE>
+hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
+  constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
+  constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
+  const KernelArgs a = make_kernel_args(p, BX, BY);
+  const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
+  if (total == 0) return hipSuccess;
+  if (hipError_t e = check_grid(total)) return e;
+  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE>;
+  static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
+  if (lds_ok != hipSuccess) return lds_ok;
   hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(NTHREADS), LDS_BYTES, stream, a);
   return hipGetLastError();
 }
 
 template <int DT, int TOUT>
 hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
-  constexpr int KT = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  if (p.variant == kOpt) {
+    if constexpr (KPM == 1) {
+      // 16-bit input: 256 x 128 block, 8 waves (two per SIMD), 3-slot ring
+      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2>(p, stream);
+    } else {
+      // fp8: an MFMA eats two K tiles; 128 x 128 block, 4 waves, 4-slot ring
+      return launch_dtl<DT, TOUT, 128, 128, 64, 64, 4, 1>(p, stream);
+    }
+  }
   // fp8 stages are twice as large (two K tiles per MFMA): one block per CU,
   // one wave per SIMD with the full register file
-  constexpr int WPE = (KT == 2) ? 1 : 2;
-  if (p.variant == kOpt) {
-    return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadTiled, WPE>(p, stream);
-  }
+  constexpr int WPE = (KPM == 2) ? 1 : 2;
   const size_t k_bytes = (size_t)p.k * bits_of(p.type_in) / 8;
   const bool aligned = (k_bytes >= 16) && (k_bytes % 16 == 0) && ((uintptr_t)p.x % 16 == 0) &&
                        ((uintptr_t)p.y % 16 == 0);
   if (aligned) {
-    return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadPlanarVec, WPE>(p, stream);
+    return launch_config<DT, TOUT, 128, 128, 64, 64, KPM, kLoadPlanarVec, WPE>(p, stream);
   }
-  return launch_config<DT, TOUT, 128, 128, 64, 64, KT, kLoadPlanarElem, WPE>(p, stream);
+  return launch_config<DT, TOUT, 128, 128, 64, 64, KPM, kLoadPlanarElem, WPE>(p, stream);
 }
 
 }  // namespace
