@@ -229,6 +229,51 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
   }
 }
 
+// Epilogue through LDS for the common case (planar fp32 C, beta = 0, wave tile
+// entirely inside C, 64 columns wide): the accumulators of 16 rows are written
+// to a wave-private LDS patch and read back row-wise, so that every store
+// instruction writes four contiguous 256-byte row segments instead of sixteen
+// 64-byte ones. `patch` is 16 rows of 272 bytes (the 16-byte pad keeps both
+// the column-wise writes and the row-wise reads free of bank conflicts).
+constexpr int kStagePatchBytes = 16 * 272;
+
+template <int TX, int TY>
+__device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, unsigned b,
+                                                       unsigned x_wave, unsigned y_wave, int lane,
+                                                       char *patch, float4_t (&acc_re)[TY][TX],
+                                                       float4_t (&acc_im)[TY][TX]) {
+  static_assert(TX == 4, "patch rows hold 64 columns");
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha;
+  const float ar = args.alpha_re, ai = args.alpha_im;
+  float *cbase = reinterpret_cast<float *>(args.c) + (size_t)b * 2 * nx * ny;
+  char *wr = patch + (lane & 15) * 272 + (lane >> 4) * 16;   // [y = lane%16][x = (lane/16)*4 ..]
+  const char *rd = patch + (lane >> 4) * 272 + (lane & 15) * 16;  // [row lane/16][x = (lane%16)*4 ..]
+  float *out = cbase + (size_t)(y_wave + (lane >> 4)) * nx + x_wave + (lane & 15) * 4;
+#pragma unroll
+  for (int plane = 0; plane < 2; ++plane) {
+#pragma unroll
+    for (int j = 0; j < TY; ++j) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i) {
+        float4_t v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float re = acc_re[j][i][e], im = acc_im[j][i][e];
+          v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
+                            : (have_alpha ? ai * re + ar * im : im);
+        }
+        *reinterpret_cast<float4_t *>(wr + i * 64) = v;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float4_t v = *reinterpret_cast<const float4_t *>(rd + r * 4 * 272);
+        *reinterpret_cast<float4_t *>(out + (size_t)plane * nx * ny + (size_t)(j * 16 + r * 4) * nx) = v;
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Register-staged kernel: global -> registers -> LDS, two LDS stages. Used for
 // the planar (basic) layouts, whose loads need bounds checks and zero fill.
@@ -358,9 +403,14 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
 // LDS is a ring of SLOTS K tiles. Iteration i waits for its own tile(s) with
 // s_waitcnt vmcnt(n) - n being the loads issued for later iterations - then
 // passes one barrier, issues the loads LEAD iterations ahead into the slot(s)
-// that the previous iteration just released, and does the math. Loads past
-// the end of K are pointed at a zero tile so that the count of outstanding
-// loads is the same in every iteration.
+// that the previous iteration just released, and does the math.
+//
+// Blocks are persistent: each walks a sequence of C tiles, and the copy simply
+// runs on into the next C tile, so its first K tiles are in flight while the
+// current tile's results are stored, and those stores drain under the next
+// tile's math. Loads past the end of K (an odd fp8 tile count) or past the
+// last C tile are pointed at a zero tile, which keeps the number of
+// outstanding loads the same in every iteration.
 // ---------------------------------------------------------------------------
 __device__ __attribute__((aligned(256))) char g_zero_tile[kTileBytes];
 
@@ -401,16 +451,17 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wx = wave % NWX, wy = wave / NWX;
-
-  const TileCoord tc = tile_coord(args, blockIdx.x);
-  const unsigned b = tc.b, block_x = tc.block_x, block_y = tc.block_y;
   const unsigned k_tiles = args.k_tiles;
+  const unsigned k_tiles_padded = (k_tiles + KPM - 1) / KPM * KPM;
+  const unsigned total = args.blocks_x * args.blocks_y * args.batch;
 
   // ---- this wave's share of the copy: LPW row blocks of every K tile ------
-  // row block q of a slot: X re, X im, Y re, Y im, 16 rows each
-  const char *src[LPW];        // wave-uniform: start of the operand tile row (K tile 0)
-  unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
+  // Row block q of a slot: X re, X im, Y re, Y im, 16 rows each. What depends
+  // on the lane (its row and swizzled chunk inside the row block) is the same
+  // for every C tile; the wave-uniform tile pointers are set per C tile.
   unsigned lane_off[LPW];      // per lane: where this lane's 16 bytes come from
+  unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
+  const char *src[LPW];        // wave-uniform: K tile 0 of the operand tile
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
   {
     const int r = lane >> 2;                                  // row inside the row block
@@ -422,62 +473,111 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       const int qq = is_x ? q : q - X_ROW_BLOCKS;
       const int rows = is_x ? BX : BY;
       const int plane = qq / (rows / 16), rb = qq % (rows / 16);
-      const unsigned row0 = (is_x ? block_x * BX : block_y * BY) + rb * 16;
-      const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
-      unsigned tile = row0 / kTileRows;
-      tile = tile < tiles ? tile : tiles - 1;   // rows past the end: any valid data, never stored
-      const char *op = is_x ? args.x + (size_t)b * args.x_batch_bytes
-                            : args.y + (size_t)b * args.y_batch_bytes;
-      src[i] = op + (size_t)tile * k_tiles * kTileBytes;
-      lane_off[i] = plane * kTilePlaneBytes + ((row0 % kTileRows) + r) * kTileRowBytes + c * 16;
+      lane_off[i] = plane * kTilePlaneBytes + (((rb * 16) % kTileRows) + r) * kTileRowBytes + c * 16;
       lds_dst[i] = lds_base + q * 1024;
     }
   }
-  auto issue = [&](unsigned kt, int slot) {
+  // The copy runs LEAD iterations ahead of the math and walks the same
+  // sequence of C tiles; past the last one it reads the zero tile.
+  unsigned load_tile = blockIdx.x, load_kt = 0;
+  auto point_at = [&](unsigned vt) {
+    if (vt < total) {
+      const TileCoord tc = tile_coord(args, vt);
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        const int q = i * NW + wave;
+        const bool is_x = q < X_ROW_BLOCKS;
+        const int qq = is_x ? q : q - X_ROW_BLOCKS;
+        const int rb = qq % ((is_x ? BX : BY) / 16);
+        const unsigned row0 = (is_x ? tc.block_x * BX : tc.block_y * BY) + rb * 16;
+        const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
+        unsigned tile = row0 / kTileRows;
+        tile = tile < tiles ? tile : tiles - 1;   // rows past the end: never stored
+        const char *op = is_x ? args.x + (size_t)tc.b * args.x_batch_bytes
+                              : args.y + (size_t)tc.b * args.y_batch_bytes;
+        src[i] = op + (size_t)tile * k_tiles * kTileBytes;
+      }
+    }
+  };
+  auto issue_next = [&](int slot) {
+    const bool real = (load_tile < total) && (load_kt < k_tiles);
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-      const char *base = kt < k_tiles ? src[i] + (size_t)kt * kTileBytes : g_zero_tile;
+      const char *base = real ? src[i] + (size_t)load_kt * kTileBytes : g_zero_tile;
       load_1k_to_lds(base, lane_off[i], lds_dst[i] + slot * SLOT_BYTES);
+    }
+    if (++load_kt == k_tiles_padded) {
+      load_kt = 0;
+      load_tile += gridDim.x;
+      point_at(load_tile);
     }
   };
 
-  float4_t acc_re[TY][TX], acc_im[TY][TX];
-#pragma unroll
-  for (int j = 0; j < TY; ++j) {
-#pragma unroll
-    for (int i = 0; i < TX; ++i) {
-      acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
-      acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    }
-  }
   const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
   const int x_frag_off = (wx * WX) * kTileRowBytes + frag_lane_off;
   const int y_frag_off = X_BYTES + (wy * WY) * kTileRowBytes + frag_lane_off;
+  // wide stores through LDS: planar C, no beta term, vector-aligned rows
+  const bool staged_ok = !args.c_interleaved && !args.have_beta && args.c_vector_ok &&
+                         (args.nx % 4 == 0);
 
   // ---- pipeline ----------------------------------------------------------
-  const unsigned iters = (k_tiles + KPM - 1) / KPM;
+  point_at(load_tile);
 #pragma unroll
-  for (int t = 0; t < LEAD * KPM; ++t) issue(t, t);
+  for (int t = 0; t < LEAD * KPM; ++t) issue_next(t);
   unsigned slot = 0;                       // first slot of the current iteration
-  for (unsigned it = 0; it < iters; ++it) {
-    wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
-    // the slots of iteration it-1 are free now: refill them for iteration it+LEAD
-    unsigned refill = slot + LEAD * KPM;
-    refill = refill >= SLOTS ? refill - SLOTS : refill;
+  const unsigned iters = k_tiles_padded / KPM;
+  for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
+    float4_t acc_re[TY][TX], acc_im[TY][TX];
 #pragma unroll
-    for (int u = 0; u < KPM; ++u) issue((it + LEAD) * KPM + u, refill + u);
-    const char *tile[KPM];
+    for (int j = 0; j < TY; ++j) {
 #pragma unroll
-    for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
-    mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
-    slot += KPM;
-    slot = slot >= SLOTS ? slot - SLOTS : slot;
+      for (int i = 0; i < TX; ++i) {
+        acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+        acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    for (unsigned it = 0; it < iters; ++it) {
+      wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
+      // the slots of the previous iteration are free now: refill them with the
+      // K tiles that are LEAD iterations ahead (of this C tile or the next)
+      unsigned refill = slot + LEAD * KPM;
+      refill = refill >= SLOTS ? refill - SLOTS : refill;
+#pragma unroll
+      for (int u = 0; u < KPM; ++u) issue_next(refill + u);
+      const char *tile[KPM];
+#pragma unroll
+      for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
+      mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
+      slot += KPM;
+      slot = slot >= SLOTS ? slot - SLOTS : slot;
+    }
+    // The stores below are not waited for here: they drain while the next C
+    // tile, whose first K tiles are already on their way, is being computed.
+    const TileCoord tc = tile_coord(args, vt);
+    const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
+    bool staged = false;
+    if constexpr (TOUT == kFloat32 && TX == 4 && NW * kStagePatchBytes <= SLOT_BYTES) {
+      if (staged_ok) {
+        // The slot consumed last is free until the next refill, but other waves
+        // may still be reading it: one barrier, then every wave uses its own
+        // patch of it. (Uniform per block, so the barrier is safe.)
+        unsigned free_slot = slot + LEAD * KPM;
+        free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
+        asm volatile("s_barrier" ::: "memory");
+        if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
+          store_wave_tile_staged<TX, TY>(args, tc.b, x_wave, y_wave, lane,
+                                         lds + free_slot * SLOT_BYTES + wave * kStagePatchBytes,
+                                         acc_re, acc_im);
+          staged = true;
+        }
+      }
+    }
+    if (!staged) {
+      store_wave_tile<TOUT, TX, TY>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+    }
   }
   // nothing may still be writing into LDS when the block gives it back
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
-  store_wave_tile<TOUT, TX, TY>(args, b, block_x * BX + wx * WX, block_y * BY + wy * WY, lane,
-                                acc_re, acc_im);
 }
 
 inline hipError_t check_grid(size_t total) {
@@ -506,10 +606,29 @@ hipError_t launch_config(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Number of compute units of the current device (queried once).
+inline int compute_units() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0) {
+      cus = 256;
+    }
+    return cus;
+  }();
+  return n;
+}
+
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
   constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
+  constexpr int kLdsPerCu = 160 * 1024;
+  constexpr int BLOCKS_PER_CU = (kLdsPerCu / LDS_BYTES) < (WPE * 256 / NTHREADS)
+                                    ? (kLdsPerCu / LDS_BYTES)
+                                    : (WPE * 256 / NTHREADS);
+  static_assert(BLOCKS_PER_CU >= 1, "configuration does not fit a CU");
   const KernelArgs a = make_kernel_args(p, BX, BY);
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
@@ -517,7 +636,11 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE>;
   static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
   if (lds_ok != hipSuccess) return lds_ok;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(NTHREADS), LDS_BYTES, stream, a);
+  // persistent blocks: as many as are resident at once, each walking C tiles
+  // with a stride of the grid size (a multiple of the XCD count)
+  const size_t resident = (size_t)compute_units() * BLOCKS_PER_CU / kNumXcd * kNumXcd;
+  const unsigned grid = (unsigned)(total < resident ? total : resident);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NTHREADS), LDS_BYTES, stream, a);
   return hipGetLastError();
 }
 
