@@ -66,6 +66,8 @@ def main():
     ap.add_argument("--workload", default="beamformer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--isolated", action="store_true",
+                    help="also time the GEMM launched back to back outside the step")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the batch axis "
@@ -107,23 +109,39 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    # Timed region: `steps` passes, bracketed by synchronisation for the wall-clock
+    # figure. Inside it every kernel is also bracketed by events recorded on the
+    # stream the kernels are launched on, which gives each kernel's duration in
+    # the situation that counts (the GEMM right after the transposes).
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        ev[i][0].record()
+        tr_a.Run(a_il.data_ptr(), a_t.data_ptr())
+        ev[i][1].record()
+        tr_b.Run(b_il.data_ptr(), b_t.data_ptr())
+        ev[i][2].record()
+        gemm.Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
+        ev[i][3].record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     flops = 8.0 * B * M * N * K
     value = flops / (ms_per_step * 1e-3) / 1e12
-
-    # per-kernel timings on the launch stream
-    iters = max(args.steps, 10)
-    gemm_ms = time_kernel(lambda: gemm.Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr()), iters, torch)
-    tra_ms = time_kernel(lambda: tr_a.Run(a_il.data_ptr(), a_t.data_ptr()), iters, torch)
-    trb_ms = time_kernel(lambda: tr_b.Run(b_il.data_ptr(), b_t.data_ptr()), iters, torch)
+    tra_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    trb_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    gemm_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
     gemm_tflops = flops / (gemm_ms * 1e-3) / 1e12
     trb_bytes = 2.0 * B * 2 * N * K * 2      # read + write, reference's definition
     tra_bytes = 2.0 * B * 2 * M * K * 2
+
+    isolated = None
+    if args.isolated:
+        # the GEMM launched back to back on its own (inputs and caches warm)
+        iters = max(args.steps, 10)
+        iso_ms = time_kernel(lambda: gemm.Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr()), iters, torch)
+        isolated = {"gemm_ms": iso_ms, "gemm_tflops": flops / (iso_ms * 1e-3) / 1e12}
 
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "gemm_f16_beamformer_traffic.json")
@@ -149,6 +167,8 @@ def main():
                     "transpose_b_ms": trb_ms, "transpose_b_gbs": trb_bytes / trb_ms / 1e6,
                     "transpose_b_frac_of_hbm_peak": trb_bytes / trb_ms / 1e6 / HBM_PEAK_GBS},
     }
+    if isolated:
+        result["isolated"] = isolated
 
     if not args.no_check:
         # one batch against a float64 product computed by an independent library

@@ -1,0 +1,8 @@
+// Umbrella header of the ccglib-compatible C++ API for gfx950.
+#ifndef CCGLIB_CCGLIB_HPP_
+#define CCGLIB_CCGLIB_HPP_
+#include <ccglib/gemm/mma.h>
+#include <ccglib/packing/packing.h>
+#include <ccglib/pipeline/pipeline.h>
+#include <ccglib/transpose/transpose.h>
+#endif
