@@ -66,6 +66,8 @@ def main():
     ap.add_argument("--workload", default="beamformer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 1 GiB device copy (for scaling rocprofv3 HBM counters)")
     ap.add_argument("--isolated", action="store_true",
                     help="also time the GEMM launched back to back outside the step")
     args = ap.parse_args()
@@ -109,6 +111,15 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    if args.copy_calibration:
+        # a copy kernel of known size: reads 1 GiB and writes 1 GiB per launch
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # Timed region: `steps` passes, bracketed by synchronisation for the wall-clock
     # figure. Inside it every kernel is also bracketed by events recorded on the
