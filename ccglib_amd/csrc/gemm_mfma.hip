@@ -537,7 +537,15 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     for (unsigned it = 0; it < iters; ++it) {
-      wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
+      // After the first C tile, the K tiles of the first LEAD iterations were
+      // already waited for before the previous epilogue (see below), so these
+      // iterations only need the barrier; waiting on the counter here would
+      // wait for the previous tile's C stores, which are younger than them.
+      if (vt != blockIdx.x && it < (unsigned)LEAD) {
+        asm volatile("s_barrier" ::: "memory");
+      } else {
+        wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
+      }
       // the slots of the previous iteration are free now: refill them with the
       // K tiles that are LEAD iterations ahead (of this C tile or the next)
       unsigned refill = slot + LEAD * KPM;
@@ -552,7 +560,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       slot = slot >= SLOTS ? slot - SLOTS : slot;
     }
     // The stores below are not waited for here: they drain while the next C
-    // tile, whose first K tiles are already on their way, is being computed.
+    // tile is being computed. The counter cannot tell loads from stores, so
+    // the next tile's first K tiles, which are already on their way, are waited
+    // for now; the first wait that has to include the stores then comes LEAD
+    // iterations into the next tile.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const TileCoord tc = tile_coord(args, vt);
     const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
     bool staged = false;
@@ -652,8 +664,9 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
       // 16-bit input: 256 x 128 block, 8 waves (two per SIMD), 3-slot ring
       return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2>(p, stream);
     } else {
-      // fp8: an MFMA eats two K tiles; 128 x 128 block, 4 waves, 4-slot ring
-      return launch_dtl<DT, TOUT, 128, 128, 64, 64, 4, 1>(p, stream);
+      // fp8: an MFMA eats two K tiles, so the ring holds 4 slots of 32 KiB;
+      // 128 x 128 block, 8 waves of 64 x 32 (two per SIMD)
+      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2>(p, stream);
     }
   }
   // fp8 stages are twice as large (two K tiles per MFMA): one block per CU,
