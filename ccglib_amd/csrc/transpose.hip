@@ -6,8 +6,9 @@
 // thread. This one is bandwidth-shaped: a thread moves 16-byte vectors (both
 // planes of 4 rows), lanes of a wave run along N across tile boundaries, so
 // loads are contiguous runs of 256 bytes per row and stores are contiguous
-// runs of rows inside each output tile. A scalar kernel covers shapes whose
-// rows are not whole 16-byte vectors.
+// runs of rows inside each output tile. Both sides are streamed once, so the
+// accesses carry the non-temporal hint (measured +5 to +10 % on this part).
+// A scalar kernel covers shapes whose rows are not whole 16-byte vectors.
 #include "common.h"
 
 namespace ccglib_amd {
@@ -74,12 +75,12 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
     if (m < a.m && n_ok) {
       if constexpr (!INTERLEAVED) {
         const char *p = a.in + (((b * 2) * a.m + m) * a.n + n0) * EB;
-        re[i] = *reinterpret_cast<const uint4_t *>(p);
-        im[i] = *reinterpret_cast<const uint4_t *>(p + a.m * a.n * EB);
+        re[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
+        im[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p + a.m * a.n * EB));
       } else {
         const char *p = a.in + ((b * a.m + m) * a.n + n0) * 2 * EB;
-        const uint4_t x = *reinterpret_cast<const uint4_t *>(p);
-        const uint4_t y = *reinterpret_cast<const uint4_t *>(p + 16);
+        const uint4_t x = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
+        const uint4_t y = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p + 16));
         deinterleave<EB>(x, y, re[i], im[i]);
       }
     }
@@ -91,8 +92,8 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
       const size_t mt = m / a.m_chunk, mr = m % a.m_chunk;
       char *q = a.out + (((b * a.m_tiles + mt) * a.n_tiles + nt) * 2) * plane_bytes +
                 (mr * a.n_chunk) * EB + v * 16;
-      *reinterpret_cast<uint4_t *>(q) = re[i];
-      *reinterpret_cast<uint4_t *>(q + plane_bytes) = im[i];
+      __builtin_nontemporal_store(re[i], reinterpret_cast<uint4_t *>(q));
+      __builtin_nontemporal_store(im[i], reinterpret_cast<uint4_t *>(q + plane_bytes));
     }
   }
 }
