@@ -97,8 +97,8 @@ class _Handle:
 
     def __del__(self):
         h = getattr(self, "_h", None)
-        if h is not None and h.value:
-            getattr(_capi.load(), self._destroy)(h)
+        if h is not None and h.value and _capi is not None and ctypes is not None:
+            getattr(_capi.load(), self._destroy)(h)   # (modules are None at interpreter exit)
             self._h = ctypes.c_void_p()
 
 

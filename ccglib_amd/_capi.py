@@ -3,7 +3,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libccglib_amd.so")
+# CCGLIB_AMD_LIBRARY may point at another build of the same library
+LIB_PATH = os.environ.get("CCGLIB_AMD_LIBRARY") or os.path.join(HERE, "libccglib_amd.so")
 
 _sz, _vp, _i, _f = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 _pvp = ctypes.POINTER(ctypes.c_void_p)
