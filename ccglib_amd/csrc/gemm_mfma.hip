@@ -276,7 +276,8 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
 
 // ---------------------------------------------------------------------------
 // Register-staged kernel: global -> registers -> LDS, two LDS stages. Used for
-// the planar (basic) layouts, whose loads need bounds checks and zero fill.
+// planar (basic) input whose rows are not whole aligned 16-byte chunks: its
+// element-wise loads do the bounds checks and the zero fill.
 // ---------------------------------------------------------------------------
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WAVES_PER_EU>
 __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma(
@@ -392,8 +393,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
 }
 
 // ---------------------------------------------------------------------------
-// Direct-to-LDS kernel for the tiled (opt) layout. Operand tiles are contiguous
-// 16 KiB blocks, so the copy into LDS needs no registers: every wave issues
+// Direct-to-LDS kernel for the tiled (opt) layout, and for planar input with
+// 16-byte aligned rows (where each lane brings its own address instead of an
+// offset into a contiguous tile). Operand tiles of the tiled layout are
+// contiguous 16 KiB blocks; the copy into LDS needs no registers: every wave issues
 // global_load_lds_dwordx4, each of which moves 16 rows x 64 bytes (1 KiB)
 // straight into LDS. The hardware writes lane L's 16 bytes at LDS offset
 // base + 16 L; the XOR swizzle of the LDS layout is obtained by letting lane L
@@ -430,7 +433,20 @@ __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_o
       : "memory");
 }
 
-template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU>
+// Same, with a full address per lane (planar layout: the 16 rows of a row block
+// are not contiguous in memory).
+__device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
+                                                       unsigned lds_address) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off"
+      :
+      : "s"(lds_address), "v"(lane_address)
+      : "memory");
+}
+
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER>
 __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma_dtl(
     const KernelArgs args) {
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
@@ -462,10 +478,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   unsigned lane_off[LPW];      // per lane: where this lane's 16 bytes come from
   unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
   const char *src[LPW];        // wave-uniform: K tile 0 of the operand tile
+  const char *lane_src[LPW];   // planar layout: this lane's chunk of K tile 0
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
+  const int r = lane >> 2;                                    // row inside the row block
+  const int c = (lane & 3) ^ ((r >> 1) & 3);                  // chunk that belongs at lane*16
   {
-    const int r = lane >> 2;                                  // row inside the row block
-    const int c = (lane & 3) ^ ((r >> 1) & 3);                // chunk that belongs at lane*16
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
       const int q = i * NW + wave;
@@ -488,23 +505,42 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         const int q = i * NW + wave;
         const bool is_x = q < X_ROW_BLOCKS;
         const int qq = is_x ? q : q - X_ROW_BLOCKS;
-        const int rb = qq % ((is_x ? BX : BY) / 16);
+        const int rows = is_x ? BX : BY;
+        const int plane = qq / (rows / 16), rb = qq % (rows / 16);
         const unsigned row0 = (is_x ? tc.block_x * BX : tc.block_y * BY) + rb * 16;
-        const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
-        unsigned tile = row0 / kTileRows;
-        tile = tile < tiles ? tile : tiles - 1;   // rows past the end: never stored
         const char *op = is_x ? args.x + (size_t)tc.b * args.x_batch_bytes
                               : args.y + (size_t)tc.b * args.y_batch_bytes;
-        src[i] = op + (size_t)tile * k_tiles * kTileBytes;
+        if constexpr (LOADER == kLoadTiled) {
+          const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
+          unsigned tile = row0 / kTileRows;
+          tile = tile < tiles ? tile : tiles - 1;   // rows past the end: never stored
+          src[i] = op + (size_t)tile * k_tiles * kTileBytes;
+        } else {
+          const unsigned total_rows = is_x ? args.nx : args.ny;
+          unsigned row = row0 + r;
+          row = row < total_rows ? row : total_rows - 1;   // likewise
+          lane_src[i] = op + ((size_t)plane * total_rows + row) * args.k_bytes + c * 16;
+        }
       }
     }
   };
   auto issue_next = [&](int slot) {
     const bool real = (load_tile < total) && (load_kt < k_tiles);
+    if constexpr (LOADER == kLoadTiled) {
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const char *base = real ? src[i] + (size_t)load_kt * kTileBytes : g_zero_tile;
-      load_1k_to_lds(base, lane_off[i], lds_dst[i] + slot * SLOT_BYTES);
+      for (int i = 0; i < LPW; ++i) {
+        const char *base = real ? src[i] + (size_t)load_kt * kTileBytes : g_zero_tile;
+        load_1k_to_lds(base, lane_off[i], lds_dst[i] + slot * SLOT_BYTES);
+      }
+    } else {
+      // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
+      const bool inside = real && (load_kt * kTileRowBytes + c * 16 + 16 <= args.k_bytes);
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        const char *p = inside ? lane_src[i] + (size_t)load_kt * kTileRowBytes
+                               : g_zero_tile + lane * 16;
+        load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
+      }
     }
     if (++load_kt == k_tiles_padded) {
       load_kt = 0;
@@ -632,7 +668,8 @@ inline int compute_units() {
   return n;
 }
 
-template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE>
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
+          int LOADER = kLoadTiled>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
   constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
@@ -645,7 +682,7 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE>;
+  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER>;
   static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
   if (lds_ok != hipSuccess) return lds_ok;
   // persistent blocks: as many as are resident at once, each walking C tiles
@@ -659,25 +696,28 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
 template <int DT, int TOUT>
 hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
-  if (p.variant == kOpt) {
+  const size_t k_bytes = (size_t)p.k * bits_of(p.type_in) / 8;
+  // planar rows made of whole, aligned 16-byte chunks can be copied straight
+  // into LDS as well; anything else goes through the register-staged kernel
+  const bool planar_direct = (p.variant == kBasic) && (k_bytes >= 16) && (k_bytes % 16 == 0) &&
+                             ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.y % 16 == 0);
+  if (p.variant == kOpt || planar_direct) {
     if constexpr (KPM == 1) {
-      // 16-bit input: 256 x 128 block, 8 waves (two per SIMD), 3-slot ring
-      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2>(p, stream);
+      // 16-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
+      return p.variant == kOpt
+                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled>(p, stream)
+                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec>(p, stream);
     } else {
       // fp8: an MFMA eats two K tiles, so the ring holds 4 slots of 32 KiB;
       // 128 x 128 block, 8 waves of 64 x 32 (two per SIMD)
-      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2>(p, stream);
+      return p.variant == kOpt
+                 ? launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadTiled>(p, stream)
+                 : launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadPlanarVec>(p, stream);
     }
   }
-  // fp8 stages are twice as large (two K tiles per MFMA): one block per CU,
-  // one wave per SIMD with the full register file
+  // fp8 stages are twice as large (two K tiles per MFMA): one wave per SIMD
+  // with the full register file
   constexpr int WPE = (KPM == 2) ? 1 : 2;
-  const size_t k_bytes = (size_t)p.k * bits_of(p.type_in) / 8;
-  const bool aligned = (k_bytes >= 16) && (k_bytes % 16 == 0) && ((uintptr_t)p.x % 16 == 0) &&
-                       ((uintptr_t)p.y % 16 == 0);
-  if (aligned) {
-    return launch_config<DT, TOUT, 128, 128, 64, 64, KPM, kLoadPlanarVec, WPE>(p, stream);
-  }
   return launch_config<DT, TOUT, 128, 128, 64, 64, KPM, kLoadPlanarElem, WPE>(p, stream);
 }
 
