@@ -97,6 +97,9 @@ struct ccglib_gemm {
   hipStream_t stream;
   int type_in, type_out, variant, c_axis, c_order;
   float alpha_re, alpha_im, beta_re, beta_im;
+  // Set by the pipeline only: A and B are the caller's interleaved (re, im)
+  // rows and are consumed as they are, without a transpose.
+  bool input_interleaved = false;
 };
 
 struct ccglib_transpose {
@@ -221,7 +224,17 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   p.c = d_c;
   p.batch = (unsigned)g->B;
   p.k = (unsigned)g->K;
-  p.k_tiles = (unsigned)ceil_div(g->K, (size_t)k_per_tile(g->type_in));
+  p.input_interleaved = g->input_interleaved;
+  if (g->input_interleaved) {
+    // a row holds K (re, im) pairs: twice the bytes, walked in 64-byte pieces
+    p.k_tiles = (unsigned)ceil_div(2 * g->K, (size_t)k_per_tile(g->type_in));
+    if ((uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0) {
+      return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                  "interleaved pipeline input must be 16-byte aligned");
+    }
+  } else {
+    p.k_tiles = (unsigned)ceil_div(g->K, (size_t)k_per_tile(g->type_in));
+  }
   if (p.k_tiles == 0) p.k_tiles = 1;  // K = 0: one all-zero tile keeps the epilogue uniform
   p.x_tiles = (unsigned)ceil_div(p.nx, kTileRows);
   p.y_tiles = (unsigned)ceil_div(p.ny, kTileRows);
@@ -448,6 +461,11 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   if (!is_enum01(input_complex_axis_location) || !is_enum01(variant)) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
   }
+  if (variant == kBasic && output_complex_axis_location == kInterleaved) {
+    // as the GEMM it wraps (src/mma/GEMM.cpp:77-80)
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "complex-interleaved output is not supported in basic variant");
+  }
   ccglib_pipeline *p = new (std::nothrow) ccglib_pipeline;
   if (!p) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
   p->B = B;
@@ -462,7 +480,13 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   p->need_copyin_c = (beta_re != 0.0f || beta_im != 0.0f);  // src/pipeline/Pipeline.cpp:138
   int rc = CCGLIB_OK;
   const bool packing = (input_type == kInt1);   // src/pipeline/Pipeline.cpp:52
-  const bool transposing = (variant == kOpt);   // :53
+  // Interleaved 8/16-bit input whose rows are whole 16-byte chunks is fed to the
+  // GEMM as it is (the kernel de-interleaves in its arithmetic), which saves the
+  // two transposes and their intermediate buffers for either variant.
+  const size_t in_bits = (size_t)bits_of(input_type);
+  const bool fused = !packing && input_complex_axis_location == kInterleaved && K > 0 &&
+                     (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0;
+  const bool transposing = (variant == kOpt) && !fused;   // :53
   // Packing already moves all real samples in front of all imaginary ones
   // (over the whole buffer), so what follows it sees planar data.
   const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
@@ -504,8 +528,10 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
       }
     }
     rc = ccglib_gemm_create(&p->gemm, B, M, N, K, device, stream, input_type, output_type,
-                            variant, output_complex_axis_location, c_mem_order, a_mem_order,
-                            b_mem_order, alpha_re, alpha_im, beta_re, beta_im);  // :102-105
+                            fused ? (int)kOpt : variant, output_complex_axis_location,
+                            c_mem_order, a_mem_order, b_mem_order, alpha_re, alpha_im, beta_re,
+                            beta_im);  // :102-105
+    if (rc == CCGLIB_OK) p->gemm->input_interleaved = fused;
   } while (false);
   if (rc != CCGLIB_OK) {
     const std::string keep = g_last_error;

@@ -68,6 +68,8 @@ struct GemmParams {
   unsigned x_tiles, y_tiles;  // 128-row tiles per operand (ceil)
   int type_in, type_out;
   int variant;          // kBasic: planar rows; kOpt: tiled layout
+  int input_interleaved;  // operands are rows of (re, im) pairs; k_tiles counts 64-byte
+                          // pieces of those rows (used by the pipeline only)
   int c_interleaved;    // 0 planar, 1 interleaved
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta;

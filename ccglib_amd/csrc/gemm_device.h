@@ -10,7 +10,7 @@ namespace ccglib_amd {
 
 typedef int int4_t __attribute__((ext_vector_type(4)));
 
-enum Loader { kLoadTiled = 0, kLoadPlanarVec = 1, kLoadPlanarElem = 2 };
+enum Loader { kLoadTiled = 0, kLoadPlanarVec = 1, kLoadPlanarElem = 2, kLoadInterleavedVec = 3 };
 
 constexpr int kNumXcd = 8;
 
@@ -151,7 +151,7 @@ inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
   a.y_tiles = p.y_tiles;
   a.blocks_x = (unsigned)ceil_div(p.nx, bx);
   a.blocks_y = (unsigned)ceil_div(p.ny, by);
-  if (p.variant == kOpt) {
+  if (p.variant == kOpt && !p.input_interleaved) {
     a.x_batch_bytes = (size_t)p.x_tiles * p.k_tiles * kTileBytes;
     a.y_batch_bytes = (size_t)p.y_tiles * p.k_tiles * kTileBytes;
   } else {

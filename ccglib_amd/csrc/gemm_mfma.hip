@@ -129,6 +129,49 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
   }
 }
 
+// The same for interleaved operands (rows of (re, im) pairs, as the caller's
+// buffers hold them). With K running over the 2K real numbers of a row,
+//   Re = sum X~ . Y1,  Y1 = (yr, -yi, ...)   and   Im = sum X~ . Y2,  Y2 = (yi, yr, ...)
+// so the raw X fragment is used as it is and both Y variants come from the raw
+// Y fragment in registers: a sign flip of the odd elements and a swap inside
+// each pair. Two MFMAs per fragment pair over half as many complex values:
+// the same MFMA and LDS work per complex MAC as with planar operands.
+template <int DT, int BX, int BY, int TX, int TY>
+__device__ __forceinline__ void mma_step_interleaved(
+    const char *const (&slot)[DtypeTraits<DT>::kTilesPerMfma], int x_frag_off, int y_frag_off,
+    float4_t (&acc_re)[TY][TX], float4_t (&acc_im)[TY][TX]) {
+  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr bool kBytes = DtypeTraits<DT>::kElemBytes == 1;
+  Fragment<DT> x[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) {
+#pragma unroll
+    for (int u = 0; u < KPM; ++u) {
+      x[i].v[u] = *reinterpret_cast<const int4_t *>(slot[u] + x_frag_off + i * 16 * kTileRowBytes);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+    Fragment<DT> y1, y2;
+#pragma unroll
+    for (int u = 0; u < KPM; ++u) {
+      const int4_t raw =
+          *reinterpret_cast<const int4_t *>(slot[u] + y_frag_off + j * 16 * kTileRowBytes);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned v = (unsigned)raw[w];
+        y1.v[u][w] = (int)(v ^ (kBytes ? 0x80008000u : 0x80000000u));
+        y2.v[u][w] = kBytes ? (int)__builtin_amdgcn_perm(v, v, 0x02030001u)
+                            : (int)__builtin_amdgcn_alignbit(v, v, 16);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(x[i], y1, acc_re[j][i]);
+#pragma unroll
+    for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(x[i], y2, acc_im[j][i]);
+  }
+}
+
 // Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
 // store. The lane holds, per 16x16 tile, x = x0 + (lane/16)*4 + 0..3 at
 // y = y0 + lane%16, i.e. four consecutive elements of the contiguous C axis.
@@ -452,15 +495,21 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
   constexpr int TX = WX / 16, TY = WY / 16;
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
-  constexpr int X_BYTES = 2 * BX * kTileRowBytes;
-  constexpr int SLOT_BYTES = X_BYTES + 2 * BY * kTileRowBytes;
+  // interleaved operands: one plane of (re, im) rows, half the work per K tile,
+  // so an iteration takes two MFMA steps to keep the barrier rate the same
+  constexpr bool IL = (LOADER == kLoadInterleavedVec);
+  constexpr int PLANES = IL ? 1 : 2;
+  constexpr int STEPS = (IL && KPM == 1) ? 2 : 1;   // MFMA steps per iteration
+  constexpr int KPI = KPM * STEPS;                  // K tiles per iteration
+  constexpr int X_BYTES = PLANES * BX * kTileRowBytes;
+  constexpr int SLOT_BYTES = X_BYTES + PLANES * BY * kTileRowBytes;
   constexpr int ROW_BLOCKS = SLOT_BYTES / 1024;     // 16 rows x 64 bytes each
   constexpr int X_ROW_BLOCKS = X_BYTES / 1024;
   static_assert(ROW_BLOCKS % NW == 0, "row blocks must divide evenly over the waves");
   constexpr int LPW = ROW_BLOCKS / NW;              // loads per wave per K tile
-  static_assert(SLOTS % KPM == 0 && SLOTS / KPM >= 2, "ring must hold at least two steps");
-  constexpr int LEAD = SLOTS / KPM - 1;             // iterations of prefetch distance
-  static_assert((LEAD - 1) * KPM * LPW < 64, "vmcnt range");
+  static_assert(SLOTS % KPI == 0 && SLOTS / KPI >= 2, "ring must hold at least two iterations");
+  constexpr int LEAD = SLOTS / KPI - 1;             // iterations of prefetch distance
+  static_assert((LEAD - 1) * KPI * LPW < 64, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -468,8 +517,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wx = wave % NWX, wy = wave / NWX;
   const unsigned k_tiles = args.k_tiles;
-  const unsigned k_tiles_padded = (k_tiles + KPM - 1) / KPM * KPM;
+  const unsigned k_tiles_padded = (k_tiles + KPI - 1) / KPI * KPI;
   const unsigned total = args.blocks_x * args.blocks_y * args.batch;
+  // bytes of one operand row in memory (planar: one plane's row)
+  const unsigned row_bytes = IL ? 2 * args.k_bytes : args.k_bytes;
 
   // ---- this wave's share of the copy: LPW row blocks of every K tile ------
   // Row block q of a slot: X re, X im, Y re, Y im, 16 rows each. What depends
@@ -519,7 +570,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           const unsigned total_rows = is_x ? args.nx : args.ny;
           unsigned row = row0 + r;
           row = row < total_rows ? row : total_rows - 1;   // likewise
-          lane_src[i] = op + ((size_t)plane * total_rows + row) * args.k_bytes + c * 16;
+          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_bytes + c * 16;
         }
       }
     }
@@ -534,7 +585,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
-      const bool inside = real && (load_kt * kTileRowBytes + c * 16 + 16 <= args.k_bytes);
+      const bool inside = real && (load_kt * kTileRowBytes + c * 16 + 16 <= row_bytes);
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
         const char *p = inside ? lane_src[i] + (size_t)load_kt * kTileRowBytes
@@ -559,9 +610,9 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   // ---- pipeline ----------------------------------------------------------
   point_at(load_tile);
 #pragma unroll
-  for (int t = 0; t < LEAD * KPM; ++t) issue_next(t);
+  for (int t = 0; t < LEAD * KPI; ++t) issue_next(t);
   unsigned slot = 0;                       // first slot of the current iteration
-  const unsigned iters = k_tiles_padded / KPM;
+  const unsigned iters = k_tiles_padded / KPI;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
     float4_t acc_re[TY][TX], acc_im[TY][TX];
 #pragma unroll
@@ -580,19 +631,26 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       if (vt != blockIdx.x && it < (unsigned)LEAD) {
         asm volatile("s_barrier" ::: "memory");
       } else {
-        wait_vmcnt_then_barrier<(LEAD - 1) * KPM * LPW>();
+        wait_vmcnt_then_barrier<(LEAD - 1) * KPI * LPW>();
       }
       // the slots of the previous iteration are free now: refill them with the
       // K tiles that are LEAD iterations ahead (of this C tile or the next)
-      unsigned refill = slot + LEAD * KPM;
+      unsigned refill = slot + LEAD * KPI;
       refill = refill >= SLOTS ? refill - SLOTS : refill;
 #pragma unroll
-      for (int u = 0; u < KPM; ++u) issue_next(refill + u);
-      const char *tile[KPM];
+      for (int u = 0; u < KPI; ++u) issue_next(refill + u);
 #pragma unroll
-      for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
-      mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
-      slot += KPM;
+      for (int st = 0; st < STEPS; ++st) {
+        const char *tile[KPM];
+#pragma unroll
+        for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + st * KPM + u) * SLOT_BYTES;
+        if constexpr (IL) {
+          mma_step_interleaved<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
+        } else {
+          mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
+        }
+      }
+      slot += KPI;
       slot = slot >= SLOTS ? slot - SLOTS : slot;
     }
     // The stores below are not waited for here: they drain while the next C
@@ -604,12 +662,12 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     const TileCoord tc = tile_coord(args, vt);
     const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
     bool staged = false;
-    if constexpr (TOUT == kFloat32 && TX == 4 && NW * kStagePatchBytes <= SLOT_BYTES) {
+    if constexpr (TOUT == kFloat32 && TX == 4 && NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
       if (staged_ok) {
         // The slot consumed last is free until the next refill, but other waves
         // may still be reading it: one barrier, then every wave uses its own
         // patch of it. (Uniform per block, so the barrier is safe.)
-        unsigned free_slot = slot + LEAD * KPM;
+        unsigned free_slot = slot + LEAD * KPI;
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
@@ -672,7 +730,8 @@ template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
           int LOADER = kLoadTiled>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
-  constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
+  constexpr int LDS_BYTES =
+      SLOTS * (LOADER == kLoadInterleavedVec ? 1 : 2) * (BX + BY) * kTileRowBytes;
   constexpr int kLdsPerCu = 160 * 1024;
   constexpr int BLOCKS_PER_CU = (kLdsPerCu / LDS_BYTES) < (WPE * 256 / NTHREADS)
                                     ? (kLdsPerCu / LDS_BYTES)
@@ -701,6 +760,15 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   // into LDS as well; anything else goes through the register-staged kernel
   const bool planar_direct = (p.variant == kBasic) && (k_bytes >= 16) && (k_bytes % 16 == 0) &&
                              ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.y % 16 == 0);
+  if (p.input_interleaved) {
+    // raw (re, im) rows straight from the caller: the host side only takes this
+    // path when the rows are whole aligned 16-byte chunks
+    if constexpr (KPM == 1) {
+      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 6, 2, kLoadInterleavedVec>(p, stream);
+    } else {
+      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 8, 2, kLoadInterleavedVec>(p, stream);
+    }
+  }
   if (p.variant == kOpt || planar_direct) {
     if constexpr (KPM == 1) {
       // 16-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring

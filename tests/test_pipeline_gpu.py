@@ -78,3 +78,45 @@ def test_pipeline_int1(variant):
     want = orc.gemm(orc.pack_bits(a_bits), orc.pack_bits(b_bits), M, N, K, orc.INT1, orc.INT32,
                     orc.ROW_MAJOR, alpha, beta, c_in)
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+
+
+def interleaved(q, B, rows, K):
+    return np.ascontiguousarray(q.reshape(B, 2, rows, K).transpose(0, 2, 3, 1)).reshape(-1)
+
+
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.float16, VT.float16),
+                                      (VT.bfloat16, VT.float32), (VT.float8e4m3, VT.float32),
+                                      (VT.float8e5m2, VT.float32)])
+@pytest.mark.parametrize("K", [4, 100, 576, 102, 33])
+@pytest.mark.parametrize("variant", [cc.Variant.opt, cc.Variant.basic])
+def test_pipeline_interleaved_input(tin, tout, K, variant):
+    # Interleaved input whose rows are whole 16-byte chunks is consumed by the GEMM
+    # directly (no transposes); other K take the transpose route (opt) - both must
+    # give the oracle's numbers. K = 102 / 33: not whole chunks.
+    if variant == cc.Variant.basic and (K * 2 * cc.Precision(tin).GetInputBits() // 8) % 16:
+        pytest.skip("the basic variant takes interleaved input only through the direct path")
+    B, M, N = 3, 200, 150
+    rng = np.random.default_rng(K)
+    qa = quantize(rng.uniform(-1, 1, B * 2 * M * K), tin)
+    qb = quantize(rng.uniform(-1, 1, B * 2 * N * K), tin)
+    alpha, beta = 0.75 - 0.5j, -0.25 + 1j
+    c32 = rng.uniform(-1, 1, B * 2 * M * N).astype(np.float32)
+    c_in = c32 if tout == VT.float32 else quantize(c32, tout)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, tin, tout,
+                    variant, alpha, beta)
+    d_a, d_b, d_c = to_device(interleaved(qa, B, M, K)), to_device(interleaved(qb, B, N, K)), to_device(c_in)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    from gpu_util import dequantize
+    got = dequantize(to_host(d_c, c_in.dtype), tout).reshape(B, 2, M, N)
+    want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], orc.ROW_MAJOR, alpha, beta, c_in)
+    w64 = orc.gemm_float64(qa, qb, M, N, K, ORC_TYPE[tin])
+    ci = dequantize(c_in, tout).reshape(B, 2, M, N).astype(np.float64)
+    w = (w64[:, 0] + 1j * w64[:, 1]) * alpha + beta * (ci[:, 0] + 1j * ci[:, 1])
+    check_float(got, dequantize(want, tout), np.stack([w.real, w.imag], 1), tin, tout)
+
+
+def test_pipeline_basic_rejects_interleaved_output():
+    with pytest.raises(RuntimeError, match="complex-interleaved output is not supported in basic variant"):
+        cc.Pipeline(1, 16, 16, 16, 0, stream(), PLANAR, INTERLEAVED, ROW, COL, ROW, VT.float16,
+                    VT.float32, cc.Variant.basic)
