@@ -85,6 +85,72 @@ __device__ __forceinline__ Fragment<DT> negate(const Fragment<DT> &f) {
   return r;
 }
 
+// The 32-row MFMAs. A lane holds 32 bytes of one row of the K tile (two
+// 16-byte chunks) and 16 accumulators per 32x32 tile. fp8 (32x32x64) eats the
+// whole 64-byte row in one instruction, 16-bit input (32x32x16) takes one
+// chunk per instruction. One wave alone keeps the MFMA pipe full with these,
+// which the 16-row shapes do not on this part (measured 58 % for 16x16x32),
+// so the second wave of a SIMD covers the other's LDS and barrier waits.
+typedef float float16_t_ __attribute__((ext_vector_type(16)));
+struct Fragment32 {
+  int4_t v[2];
+};
+
+template <int DT>
+__device__ __forceinline__ float16_t_ mfma32(const Fragment32 &a, const Fragment32 &b,
+                                             float16_t_ acc) {
+  if constexpr (DT == kFloat16) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a.v[u]),
+                                                   __builtin_bit_cast(half8_t, b.v[u]), acc, 0, 0, 0);
+    }
+    return acc;
+  } else if constexpr (DT == kBfloat16) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a.v[u]),
+                                                    __builtin_bit_cast(bf16x8_t, b.v[u]), acc, 0, 0, 0);
+    }
+    return acc;
+  } else {
+    int8_t_ av, bv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      av[i] = a.v[0][i];
+      av[4 + i] = a.v[1][i];
+      bv[i] = b.v[0][i];
+      bv[4 + i] = b.v[1][i];
+    }
+    constexpr int fmt = (DT == kFloat8e4m3) ? 0 : 1;
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, fmt, fmt, 0, 0x7f, 0,
+                                                           0x7f);
+  }
+}
+
+// Accumulator of one MFMA tile and how the output is spread over a wave, for
+// both MFMA shapes (MS = 16 or 32 rows). A lane holds "pieces" of four
+// consecutive x (the contiguous C axis) at one y:
+//   MS 16: piece (jj, ii) at x = 16 ii + 4 (lane / 16), y = 16 jj + lane % 16
+//   MS 32: piece (jj, ii) at x = 32 (ii / 4) + 8 (ii % 4) + 4 (lane / 32), y = 32 jj + lane % 32
+template <int MS> struct AccType { using type = float4_t; };
+template <> struct AccType<32> { using type = float16_t_; };
+
+template <int MS> __device__ __forceinline__ unsigned piece_x(int ii, int lane) {
+  return MS == 16 ? ii * 16 + (lane >> 4) * 4 : (ii >> 2) * 32 + (ii & 3) * 8 + (lane >> 5) * 4;
+}
+template <int MS> __device__ __forceinline__ unsigned piece_y(int jj, int lane) {
+  return MS == 16 ? jj * 16 + (lane & 15) : jj * 32 + (lane & 31);
+}
+template <int MS, typename Acc>
+__device__ __forceinline__ float piece_elem(const Acc &acc, int jj, int ii, int e) {
+  if constexpr (MS == 16) {
+    return acc[jj][ii][e];
+  } else {
+    return acc[jj][ii >> 2][(ii & 3) * 4 + e];
+  }
+}
+
 template <int TOUT> struct OutType;
 template <> struct OutType<kFloat32> { using type = float; };
 template <> struct OutType<kFloat16> { using type = _Float16; };
@@ -127,6 +193,68 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
 #pragma unroll
     for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
   }
+}
+
+// The same on the 32-row MFMAs: TX x TY tiles of 32x32, one K tile per step.
+// off[0] and off[1] are the lane's two 16-byte chunks of its row.
+template <int DT, int BX, int BY, int TX, int TY>
+__device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[2],
+                                           const int (&y_off)[2], float16_t_ (&acc_re)[TY][TX],
+                                           float16_t_ (&acc_im)[TY][TX]) {
+  constexpr int D = TX > TY ? TX : TY;
+  Fragment32 xr[TX], xi[TX], yr[TY], yi[TY], yin[TY];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    if (d < TX) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const char *p = slot + x_off[u] + d * 32 * kTileRowBytes;
+        xr[d].v[u] = *reinterpret_cast<const int4_t *>(p);
+        xi[d].v[u] = *reinterpret_cast<const int4_t *>(p + BX * kTileRowBytes);
+      }
+    }
+    if (d < TY) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const char *p = slot + y_off[u] + d * 32 * kTileRowBytes;
+        yr[d].v[u] = *reinterpret_cast<const int4_t *>(p);
+        yi[d].v[u] = *reinterpret_cast<const int4_t *>(p + BY * kTileRowBytes);
+      }
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (d < TY) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) yin[d].v[u][w] = yi[d].v[u][w] ^ (int)DtypeTraits<DT>::kSignMask;
+      }
+    }
+    int ti[TX + TY], tj[TX + TY], n = 0;
+    if (d < TX) {
+#pragma unroll
+      for (int j = 0; j < d && j < TY; ++j) ti[n] = d, tj[n] = j, ++n;
+    }
+    if (d < TY) {
+#pragma unroll
+      for (int i = 0; i <= d && i < TX; ++i) ti[n] = i, tj[n] = d, ++n;
+    }
+#pragma unroll
+    for (int t = 0; t < n; ++t)
+      acc_re[tj[t]][ti[t]] = mfma32<DT>(xr[ti[t]], yr[tj[t]], acc_re[tj[t]][ti[t]]);
+#pragma unroll
+    for (int t = 0; t < n; ++t)
+      acc_im[tj[t]][ti[t]] = mfma32<DT>(xr[ti[t]], yi[tj[t]], acc_im[tj[t]][ti[t]]);
+#pragma unroll
+    for (int t = 0; t < n; ++t)
+      acc_re[tj[t]][ti[t]] = mfma32<DT>(xi[ti[t]], yin[tj[t]], acc_re[tj[t]][ti[t]]);
+#pragma unroll
+    for (int t = 0; t < n; ++t)
+      acc_im[tj[t]][ti[t]] = mfma32<DT>(xi[ti[t]], yr[tj[t]], acc_im[tj[t]][ti[t]]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // The same for interleaved operands (rows of (re, im) pairs, as the caller's
@@ -173,13 +301,13 @@ __device__ __forceinline__ void mma_step_interleaved(
 }
 
 // Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
-// store. The lane holds, per 16x16 tile, x = x0 + (lane/16)*4 + 0..3 at
-// y = y0 + lane%16, i.e. four consecutive elements of the contiguous C axis.
-template <int TOUT, int TX, int TY>
+// store, piece by piece (four consecutive elements of the contiguous C axis).
+template <int TOUT, int TX, int TY, int MS = 16, typename Acc>
 __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned b, unsigned x_wave,
-                                                unsigned y_wave, int lane,
-                                                float4_t (&acc_re)[TY][TX],
-                                                float4_t (&acc_im)[TY][TX]) {
+                                                unsigned y_wave, int lane, const Acc &acc_re,
+                                                const Acc &acc_im) {
+  // TX, TY count MFMA tiles; pieces per tile row: 1 (MS 16) or 4 (MS 32)
+  constexpr int NPX = MS == 16 ? TX : TX * 4;
   using Tout = typename OutType<TOUT>::type;
   const unsigned nx = args.nx, ny = args.ny;
   const bool have_alpha = args.have_alpha, have_beta = args.have_beta;
@@ -188,16 +316,16 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
   const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
-    const unsigned y = y_wave + j * 16 + (lane & 15);
+    const unsigned y = y_wave + piece_y<MS>(j, lane);
 #pragma unroll
-    for (int i = 0; i < TX; ++i) {
-      const unsigned x = x_wave + i * 16 + (lane >> 4) * 4;
+    for (int i = 0; i < NPX; ++i) {
+      const unsigned x = x_wave + piece_x<MS>(i, lane);
       if (y >= ny || x >= nx) continue;
       float re[4], im[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        re[e] = acc_re[j][i][e];
-        im[e] = acc_im[j][i][e];
+        re[e] = piece_elem<MS>(acc_re, j, i, e);
+        im[e] = piece_elem<MS>(acc_im, j, i, e);
         if (have_alpha) {
           const float r0 = re[e];
           re[e] = ar * r0 - ai * im[e];
@@ -312,6 +440,51 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
       for (int r = 0; r < 4; ++r) {
         const float4_t v = *reinterpret_cast<const float4_t *>(rd + r * 4 * 272);
         *reinterpret_cast<float4_t *>(out + (size_t)plane * nx * ny + (size_t)(j * 16 + r * 4) * nx) = v;
+      }
+    }
+  }
+}
+
+// The same for the 32-row MFMA layout: one 32 x 32 tile at a time goes through
+// a patch of 32 rows of 144 bytes (128 + 16 of padding), and every store
+// instruction writes eight whole 128-byte row segments.
+constexpr int kStagePatch32Bytes = 32 * 144;
+
+template <int TX, int TY>
+__device__ __forceinline__ void store_wave_tile_staged32(const KernelArgs &args, unsigned b,
+                                                         unsigned x_wave, unsigned y_wave, int lane,
+                                                         char *patch, float16_t_ (&acc_re)[TY][TX],
+                                                         float16_t_ (&acc_im)[TY][TX]) {
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha;
+  const float ar = args.alpha_re, ai = args.alpha_im;
+  float *cbase = reinterpret_cast<float *>(args.c) + (size_t)b * 2 * nx * ny;
+  char *wr = patch + (lane & 31) * 144 + (lane >> 5) * 16;        // [y = lane%32][x = 8k + 4 (lane/32) ..]
+  const char *rd = patch + (lane >> 3) * 144 + (lane & 7) * 16;   // [row lane/8 (+8q)][x = 4 (lane%8) ..]
+  float *out = cbase + (size_t)(y_wave + (lane >> 3)) * nx + x_wave + (lane & 7) * 4;
+#pragma unroll
+  for (int plane = 0; plane < 2; ++plane) {
+#pragma unroll
+    for (int j = 0; j < TY; ++j) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float4_t v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float re = acc_re[j][i][4 * k + e], im = acc_im[j][i][4 * k + e];
+            v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
+                              : (have_alpha ? ai * re + ar * im : im);
+          }
+          *reinterpret_cast<float4_t *>(wr + k * 32) = v;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4_t v = *reinterpret_cast<const float4_t *>(rd + q * 8 * 144);
+          *reinterpret_cast<float4_t *>(out + (size_t)plane * nx * ny +
+                                        (size_t)(j * 32 + q * 8) * nx + i * 32) = v;
+        }
       }
     }
   }
@@ -489,12 +662,15 @@ __device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
       : "memory");
 }
 
-template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER>
+template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER,
+          int MS>
 __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma_dtl(
     const KernelArgs args) {
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
-  constexpr int TX = WX / 16, TY = WY / 16;
-  constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr int TX = WX / MS, TY = WY / MS;          // MFMA tiles of a wave
+  constexpr int KPM = MS == 32 ? 1 : DtypeTraits<DT>::kTilesPerMfma;
+  static_assert(MS == 16 || (MS == 32 && LOADER != kLoadInterleavedVec),
+                "the 32-row MFMAs are used for planar operands");
   // interleaved operands: one plane of (re, im) rows, half the work per K tile,
   // so an iteration takes two MFMA steps to keep the barrier rate the same
   constexpr bool IL = (LOADER == kLoadInterleavedVec);
@@ -526,13 +702,17 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   // Row block q of a slot: X re, X im, Y re, Y im, 16 rows each. What depends
   // on the lane (its row and swizzled chunk inside the row block) is the same
   // for every C tile; the wave-uniform tile pointers are set per C tile.
-  unsigned lane_off[LPW];      // per lane: where this lane's 16 bytes come from
+  unsigned tile_off[LPW];      // wave-uniform: the row block inside its operand tile
+  const unsigned lane_off = (lane >> 2) * kTileRowBytes +
+                            (((lane & 3) ^ (MS == 32 ? (lane >> 4) & 3 : (lane >> 3) & 3)) * 16);
   unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
   const char *src[LPW];        // wave-uniform: K tile 0 of the operand tile
   const char *lane_src[LPW];   // planar layout: this lane's chunk of K tile 0
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
   const int r = lane >> 2;                                    // row inside the row block
-  const int c = (lane & 3) ^ ((r >> 1) & 3);                  // chunk that belongs at lane*16
+  // chunk that belongs at lane*16: the XOR pattern that makes the fragment
+  // reads of the MFMA shape in use free of bank conflicts (measured)
+  const int c = (lane & 3) ^ (MS == 32 ? (r >> 2) & 3 : (r >> 1) & 3);
   {
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
@@ -541,7 +721,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       const int qq = is_x ? q : q - X_ROW_BLOCKS;
       const int rows = is_x ? BX : BY;
       const int plane = qq / (rows / 16), rb = qq % (rows / 16);
-      lane_off[i] = plane * kTilePlaneBytes + (((rb * 16) % kTileRows) + r) * kTileRowBytes + c * 16;
+      // inside the operand tile: the lane's part is the same for every row block
+      tile_off[i] = plane * kTilePlaneBytes + ((rb * 16) % kTileRows) * kTileRowBytes;
       lds_dst[i] = lds_base + q * 1024;
     }
   }
@@ -580,8 +761,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     if constexpr (LOADER == kLoadTiled) {
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
-        const char *base = real ? src[i] + (size_t)load_kt * kTileBytes : g_zero_tile;
-        load_1k_to_lds(base, lane_off[i], lds_dst[i] + slot * SLOT_BYTES);
+        const char *base = real ? src[i] + (size_t)load_kt * kTileBytes + tile_off[i] : g_zero_tile;
+        load_1k_to_lds(base, lane_off, lds_dst[i] + slot * SLOT_BYTES);
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
@@ -603,6 +784,15 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
   const int x_frag_off = (wx * WX) * kTileRowBytes + frag_lane_off;
   const int y_frag_off = X_BYTES + (wy * WY) * kTileRowBytes + frag_lane_off;
+  // 32-row MFMA: row lane % 32, chunks lane / 32 and lane / 32 + 2 (any split
+  // of K over the lanes is fine as long as X and Y use the same one)
+  const int row32 = lane & 31, sw32 = (row32 >> 2) & 3;
+  const int frag32_off[2] = {row32 * kTileRowBytes + (((lane >> 5) ^ sw32) * 16),
+                             row32 * kTileRowBytes + ((((lane >> 5) | 2) ^ sw32) * 16)};
+  const int x32_off[2] = {(wx * WX) * kTileRowBytes + frag32_off[0],
+                          (wx * WX) * kTileRowBytes + frag32_off[1]};
+  const int y32_off[2] = {X_BYTES + (wy * WY) * kTileRowBytes + frag32_off[0],
+                          X_BYTES + (wy * WY) * kTileRowBytes + frag32_off[1]};
   // wide stores through LDS: planar C, no beta term, vector-aligned rows
   const bool staged_ok = !args.c_interleaved && !args.have_beta && args.c_vector_ok &&
                          (args.nx % 4 == 0);
@@ -614,13 +804,13 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   unsigned slot = 0;                       // first slot of the current iteration
   const unsigned iters = k_tiles_padded / KPI;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
-    float4_t acc_re[TY][TX], acc_im[TY][TX];
+    typename AccType<MS>::type acc_re[TY][TX], acc_im[TY][TX];
 #pragma unroll
     for (int j = 0; j < TY; ++j) {
 #pragma unroll
       for (int i = 0; i < TX; ++i) {
-        acc_re[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
-        acc_im[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+        acc_re[j][i] = 0.f;
+        acc_im[j][i] = 0.f;
       }
     }
     for (unsigned it = 0; it < iters; ++it) {
@@ -644,7 +834,9 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         const char *tile[KPM];
 #pragma unroll
         for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + st * KPM + u) * SLOT_BYTES;
-        if constexpr (IL) {
+        if constexpr (MS == 32) {
+          mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im);
+        } else if constexpr (IL) {
           mma_step_interleaved<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
         } else {
           mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
@@ -662,7 +854,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     const TileCoord tc = tile_coord(args, vt);
     const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
     bool staged = false;
-    if constexpr (TOUT == kFloat32 && TX == 4 && NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
+    if constexpr (MS == 16 && TOUT == kFloat32 && TX == 4 &&
+                  NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
       if (staged_ok) {
         // The slot consumed last is free until the next refill, but other waves
         // may still be reading it: one barrier, then every wave uses its own
@@ -678,8 +871,21 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         }
       }
     }
+    if constexpr (MS == 32 && TOUT == kFloat32 && NW * kStagePatch32Bytes <= KPI * SLOT_BYTES) {
+      if (staged_ok) {
+        unsigned free_slot = slot + LEAD * KPI;
+        free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
+        asm volatile("s_barrier" ::: "memory");
+        if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
+          store_wave_tile_staged32<TX, TY>(args, tc.b, x_wave, y_wave, lane,
+                                           lds + free_slot * SLOT_BYTES + wave * kStagePatch32Bytes,
+                                           acc_re, acc_im);
+          staged = true;
+        }
+      }
+    }
     if (!staged) {
-      store_wave_tile<TOUT, TX, TY>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+      store_wave_tile<TOUT, TX, TY, MS>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
     }
   }
   // nothing may still be writing into LDS when the block gives it back
@@ -727,7 +933,7 @@ inline int compute_units() {
 }
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
-          int LOADER = kLoadTiled>
+          int LOADER = kLoadTiled, int MS = 16>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
   constexpr int LDS_BYTES =
@@ -741,7 +947,7 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER>;
+  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS>;
   static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
   if (lds_ok != hipSuccess) return lds_ok;
   // persistent blocks: as many as are resident at once, each walking C tiles
@@ -776,11 +982,11 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
                  ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled>(p, stream)
                  : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec>(p, stream);
     } else {
-      // fp8: an MFMA eats two K tiles, so the ring holds 4 slots of 32 KiB;
-      // 128 x 128 block, 8 waves of 64 x 32 (two per SIMD)
+      // fp8: the 32x32x64 MFMA takes one K tile per instruction, which lets the
+      // same block shape and ring as for 16-bit input fit into LDS
       return p.variant == kOpt
-                 ? launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadTiled>(p, stream)
-                 : launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadPlanarVec>(p, stream);
+                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
+                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
     }
   }
   // fp8 stages are twice as large (two K tiles per MFMA): one wave per SIMD
