@@ -166,6 +166,23 @@ def test_alpha_beta_narrow_output(tin, tout):
                beta=1.5 + 0.5j)
 
 
+@pytest.mark.parametrize("tin", [VT.float8e4m3, VT.float8e5m2])
+@pytest.mark.parametrize("variant,c_axis,beta", [(cc.Variant.opt, PLANAR, 0), (cc.Variant.opt, PLANAR, 0.5 - 0.25j),
+                                                 (cc.Variant.opt, INTERLEAVED, 0.5 - 0.25j),
+                                                 (cc.Variant.basic, PLANAR, 0.5 - 0.25j)])
+def test_alpha_beta_fp8(tin, variant, c_axis, beta):
+    # whole 64 x 64 wave tiles inside C (wide stores through LDS when beta is 0) and ragged ones
+    float_case(3, 256, 320, 192, tin, VT.float32, variant, c_axis, ROW, alpha=0.75 - 0.5j, beta=beta)
+    float_case(2, 200, 130, 128, tin, VT.float32, variant, c_axis, COL, alpha=-1.25j, beta=beta, seed=5)
+
+
+@pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
+def test_more_c_tiles_than_resident_blocks(tin):
+    # 1536 C tiles of 256 x 128 for at most 256 persistent blocks: every block
+    # walks several tiles, with the copy running across the tile boundaries
+    float_case(48, 256, 1024, 128, tin, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=11)
+
+
 def test_beta_zero_ignores_nan_in_c():
     # run_gemm poisons C with NaN whenever beta == 0: every float case above covers
     # it; this one states the property on its own
