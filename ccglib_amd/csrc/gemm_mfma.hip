@@ -265,38 +265,46 @@ __device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[
 // each pair. Two MFMAs per fragment pair over half as many complex values:
 // the same MFMA and LDS work per complex MAC as with planar operands.
 template <int DT, int BX, int BY, int TX, int TY>
-__device__ __forceinline__ void mma_step_interleaved(
-    const char *const (&slot)[DtypeTraits<DT>::kTilesPerMfma], int x_frag_off, int y_frag_off,
-    float4_t (&acc_re)[TY][TX], float4_t (&acc_im)[TY][TX]) {
+__device__ __forceinline__ void mma_step_interleaved(const char *slot, const int (&x_off)[2],
+                                                     const int (&y_off)[2],
+                                                     float4_t (&acc_re)[TY][TX],
+                                                     float4_t (&acc_im)[TY][TX]) {
+  // The slot holds 128 bytes of every row; x_off / y_off are the lane's two
+  // 16-byte chunks of its row. fp8 takes both in one MFMA, 16-bit input one
+  // per MFMA (two passes over the slot).
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
+  constexpr int PASSES = 2 / KPM;
   constexpr bool kBytes = DtypeTraits<DT>::kElemBytes == 1;
-  Fragment<DT> x[TX];
 #pragma unroll
-  for (int i = 0; i < TX; ++i) {
+  for (int h = 0; h < PASSES; ++h) {
+    Fragment<DT> x[TX];
 #pragma unroll
-    for (int u = 0; u < KPM; ++u) {
-      x[i].v[u] = *reinterpret_cast<const int4_t *>(slot[u] + x_frag_off + i * 16 * kTileRowBytes);
-    }
-  }
+    for (int i = 0; i < TX; ++i) {
 #pragma unroll
-  for (int j = 0; j < TY; ++j) {
-    Fragment<DT> y1, y2;
-#pragma unroll
-    for (int u = 0; u < KPM; ++u) {
-      const int4_t raw =
-          *reinterpret_cast<const int4_t *>(slot[u] + y_frag_off + j * 16 * kTileRowBytes);
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const unsigned v = (unsigned)raw[w];
-        y1.v[u][w] = (int)(v ^ (kBytes ? 0x80008000u : 0x80000000u));
-        y2.v[u][w] = kBytes ? (int)__builtin_amdgcn_perm(v, v, 0x02030001u)
-                            : (int)__builtin_amdgcn_alignbit(v, v, 16);
+      for (int u = 0; u < KPM; ++u) {
+        x[i].v[u] = *reinterpret_cast<const int4_t *>(slot + x_off[h * KPM + u] + i * 16 * 128);
       }
     }
 #pragma unroll
-    for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(x[i], y1, acc_re[j][i]);
+    for (int j = 0; j < TY; ++j) {
+      Fragment<DT> y1, y2;
 #pragma unroll
-    for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(x[i], y2, acc_im[j][i]);
+      for (int u = 0; u < KPM; ++u) {
+        const int4_t raw =
+            *reinterpret_cast<const int4_t *>(slot + y_off[h * KPM + u] + j * 16 * 128);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const unsigned v = (unsigned)raw[w];
+          y1.v[u][w] = (int)(v ^ (kBytes ? 0x80008000u : 0x80000000u));
+          y2.v[u][w] = kBytes ? (int)__builtin_amdgcn_perm(v, v, 0x02030001u)
+                              : (int)__builtin_amdgcn_alignbit(v, v, 16);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(x[i], y1, acc_re[j][i]);
+#pragma unroll
+      for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(x[i], y2, acc_im[j][i]);
+    }
   }
 }
 
@@ -671,15 +679,17 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   constexpr int KPM = MS == 32 ? 1 : DtypeTraits<DT>::kTilesPerMfma;
   static_assert(MS == 16 || (MS == 32 && LOADER != kLoadInterleavedVec),
                 "the 32-row MFMAs are used for planar operands");
-  // interleaved operands: one plane of (re, im) rows, half the work per K tile,
-  // so an iteration takes two MFMA steps to keep the barrier rate the same
+  // interleaved operands: one plane of (re, im) rows
+  // (their slots hold 128 bytes of every row, fetched as whole cache lines)
   constexpr bool IL = (LOADER == kLoadInterleavedVec);
   constexpr int PLANES = IL ? 1 : 2;
-  constexpr int STEPS = (IL && KPM == 1) ? 2 : 1;   // MFMA steps per iteration
-  constexpr int KPI = KPM * STEPS;                  // K tiles per iteration
-  constexpr int X_BYTES = PLANES * BX * kTileRowBytes;
-  constexpr int SLOT_BYTES = X_BYTES + PLANES * BY * kTileRowBytes;
-  constexpr int ROW_BLOCKS = SLOT_BYTES / 1024;     // 16 rows x 64 bytes each
+  constexpr int RB = IL ? 128 : kTileRowBytes;      // bytes of a row in one slot
+  constexpr int RPB = 1024 / RB;                    // rows moved by one 1 KiB copy instruction
+  constexpr int CPR = RB / 16;                      // 16-byte chunks per row
+  constexpr int KPI = IL ? 1 : KPM;                 // slots per iteration
+  constexpr int X_BYTES = PLANES * BX * RB;
+  constexpr int SLOT_BYTES = X_BYTES + PLANES * BY * RB;
+  constexpr int ROW_BLOCKS = SLOT_BYTES / 1024;     // 1 KiB each: 16 rows x 64 bytes or 8 x 128
   constexpr int X_ROW_BLOCKS = X_BYTES / 1024;
   static_assert(ROW_BLOCKS % NW == 0, "row blocks must divide evenly over the waves");
   constexpr int LPW = ROW_BLOCKS / NW;              // loads per wave per K tile
@@ -692,7 +702,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wx = wave % NWX, wy = wave / NWX;
-  const unsigned k_tiles = args.k_tiles;
+  // slots along K (the host counts 64-byte pieces of a row)
+  const unsigned k_tiles = IL ? (args.k_tiles + 1) / 2 : args.k_tiles;
   const unsigned k_tiles_padded = (k_tiles + KPI - 1) / KPI * KPI;
   const unsigned total = args.blocks_x * args.blocks_y * args.batch;
   // bytes of one operand row in memory (planar: one plane's row)
@@ -709,10 +720,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const char *src[LPW];        // wave-uniform: K tile 0 of the operand tile
   const char *lane_src[LPW];   // planar layout: this lane's chunk of K tile 0
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
-  const int r = lane >> 2;                                    // row inside the row block
+  const int r = lane / CPR;                                   // row inside the row block
   // chunk that belongs at lane*16: the XOR pattern that makes the fragment
   // reads of the MFMA shape in use free of bank conflicts (measured)
-  const int c = (lane & 3) ^ (MS == 32 ? (r >> 2) & 3 : (r >> 1) & 3);
+  const int c = (lane % CPR) ^ (IL ? r & 7 : MS == 32 ? (r >> 2) & 3 : (r >> 1) & 3);
   {
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
@@ -720,9 +731,9 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       const bool is_x = q < X_ROW_BLOCKS;
       const int qq = is_x ? q : q - X_ROW_BLOCKS;
       const int rows = is_x ? BX : BY;
-      const int plane = qq / (rows / 16), rb = qq % (rows / 16);
+      const int plane = qq / (rows / RPB), rb = qq % (rows / RPB);
       // inside the operand tile: the lane's part is the same for every row block
-      tile_off[i] = plane * kTilePlaneBytes + ((rb * 16) % kTileRows) * kTileRowBytes;
+      tile_off[i] = plane * kTilePlaneBytes + ((rb * RPB) % kTileRows) * kTileRowBytes;
       lds_dst[i] = lds_base + q * 1024;
     }
   }
@@ -738,8 +749,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         const bool is_x = q < X_ROW_BLOCKS;
         const int qq = is_x ? q : q - X_ROW_BLOCKS;
         const int rows = is_x ? BX : BY;
-        const int plane = qq / (rows / 16), rb = qq % (rows / 16);
-        const unsigned row0 = (is_x ? tc.block_x * BX : tc.block_y * BY) + rb * 16;
+        const int plane = qq / (rows / RPB), rb = qq % (rows / RPB);
+        const unsigned row0 = (is_x ? tc.block_x * BX : tc.block_y * BY) + rb * RPB;
         const char *op = is_x ? args.x + (size_t)tc.b * args.x_batch_bytes
                               : args.y + (size_t)tc.b * args.y_batch_bytes;
         if constexpr (LOADER == kLoadTiled) {
@@ -766,10 +777,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
-      const bool inside = real && (load_kt * kTileRowBytes + c * 16 + 16 <= row_bytes);
+      const bool inside = real && (load_kt * RB + c * 16 + 16 <= row_bytes);
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
-        const char *p = inside ? lane_src[i] + (size_t)load_kt * kTileRowBytes
+        const char *p = inside ? lane_src[i] + (size_t)load_kt * RB
                                : g_zero_tile + lane * 16;
         load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
       }
@@ -793,6 +804,13 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
                           (wx * WX) * kTileRowBytes + frag32_off[1]};
   const int y32_off[2] = {X_BYTES + (wy * WY) * kTileRowBytes + frag32_off[0],
                           X_BYTES + (wy * WY) * kTileRowBytes + frag32_off[1]};
+  // interleaved rows of 128 bytes: row lane % 16, chunks lane / 16 and lane / 16 + 4
+  const int il_row = lane & 15;
+  const int il_off[2] = {il_row * 128 + (((lane >> 4) ^ (il_row & 7)) * 16),
+                         il_row * 128 + ((((lane >> 4) | 4) ^ (il_row & 7)) * 16)};
+  const int xil_off[2] = {(wx * WX) * 128 + il_off[0], (wx * WX) * 128 + il_off[1]};
+  const int yil_off[2] = {X_BYTES + (wy * WY) * 128 + il_off[0],
+                          X_BYTES + (wy * WY) * 128 + il_off[1]};
   // wide stores through LDS: planar C, no beta term, vector-aligned rows
   const bool staged_ok = !args.c_interleaved && !args.have_beta && args.c_vector_ok &&
                          (args.nx % 4 == 0);
@@ -829,15 +847,15 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       refill = refill >= SLOTS ? refill - SLOTS : refill;
 #pragma unroll
       for (int u = 0; u < KPI; ++u) issue_next(refill + u);
-#pragma unroll
-      for (int st = 0; st < STEPS; ++st) {
+      if constexpr (IL) {
+        mma_step_interleaved<DT, BX, BY, TX, TY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
+                                                 acc_im);
+      } else {
         const char *tile[KPM];
 #pragma unroll
-        for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + st * KPM + u) * SLOT_BYTES;
+        for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
         if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im);
-        } else if constexpr (IL) {
-          mma_step_interleaved<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
         } else {
           mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
         }
@@ -936,8 +954,7 @@ template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
           int LOADER = kLoadTiled, int MS = 16>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
-  constexpr int LDS_BYTES =
-      SLOTS * (LOADER == kLoadInterleavedVec ? 1 : 2) * (BX + BY) * kTileRowBytes;
+  constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
   constexpr int kLdsPerCu = 160 * 1024;
   constexpr int BLOCKS_PER_CU = (kLdsPerCu / LDS_BYTES) < (WPE * 256 / NTHREADS)
                                     ? (kLdsPerCu / LDS_BYTES)
@@ -970,9 +987,9 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     // raw (re, im) rows straight from the caller: the host side only takes this
     // path when the rows are whole aligned 16-byte chunks
     if constexpr (KPM == 1) {
-      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 6, 2, kLoadInterleavedVec>(p, stream);
+      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec>(p, stream);
     } else {
-      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 8, 2, kLoadInterleavedVec>(p, stream);
+      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec>(p, stream);
     }
   }
   if (p.variant == kOpt || planar_direct) {
