@@ -27,9 +27,9 @@ if ROOT not in sys.path:
 # published dense peaks of MI355X
 MFMA_PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "fp8": 5033.2}
 HBM_PEAK_GBS = 8000.0
-# vector-ALU issue roof of the 1-bit GEMM: 256 CUs x 64 lane-ops/clk x 2.4 GHz, 8 lane-ops
-# (4 XOR + 4 popcount-accumulate) per 32 complex MACs, 8 "ops" per complex MAC
-INT1_VALU_ROOF_TOPS = 256 * 64 * 2.4e9 * (32 / 8) * 8 / 1e12
+# The 1-bit GEMM runs on the fp4 MFMA (operands expanded to +-1 nibbles by a
+# bandwidth-bound kernel that is part of the GEMM call): published fp4 dense peak
+FP4_PEAK_TOPS = 10066.3
 
 WORKLOADS = {
     # name: (B, M, N, K, input type, output type, input axis, description)
@@ -238,8 +238,8 @@ def main():
         per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
 
     if tin == VT.int1:
-        dtype, peak, bound, unit = "u32", INT1_VALU_ROOF_TOPS, "valu", "TOP/s"
-        kernel_name = "complex_gemm_int1<tiled>"
+        dtype, peak, bound, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "mfma", "TOP/s"
+        kernel_name = "expand_int1_to_fp4 x2 + complex_gemm_mfma_dtl<fp4->int32>"
     else:
         dtype = {"float16": "f16", "bfloat16": "bf16"}.get(tin_name, "fp8")
         peak, bound, unit = MFMA_PEAK_TFLOPS[dtype], "mfma", "TFLOP/s"

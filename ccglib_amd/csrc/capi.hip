@@ -5,6 +5,7 @@
 // src/pipeline/Pipeline.cpp.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -100,6 +101,10 @@ struct ccglib_gemm {
   // Set by the pipeline only: A and B are the caller's interleaved (re, im)
   // rows and are consumed as they are, without a transpose.
   bool input_interleaved = false;
+  // 1-bit GEMM: device memory for the operands expanded for the MFMA path
+  // (null: the popcount kernel runs instead)
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
 };
 
 struct ccglib_transpose {
@@ -204,6 +209,27 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
   g->alpha_im = alpha_im;
   g->beta_re = beta_re;
   g->beta_im = beta_im;
+  if (type_in == kInt1 && B && M && N) {
+    // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs;
+    // CCGLIB_AMD_INT1_WORKSPACE_MB caps the expanded operands (the GEMM then runs
+    // in groups of batches). Failing to get the memory is not an error.
+    const char *kernel = std::getenv("CCGLIB_AMD_INT1_KERNEL");
+    const char *cap_mb = std::getenv("CCGLIB_AMD_INT1_WORKSPACE_MB");
+    size_t bytes = gemm_int1_workspace_bytes(B, M, N, K);
+    const size_t per_batch = bytes / B;
+    size_t cap = cap_mb ? (size_t)std::strtoull(cap_mb, nullptr, 10) << 20 : (size_t)16 << 30;
+    if (cap < per_batch) cap = per_batch;
+    if (bytes > cap) bytes = cap / per_batch * per_batch;
+    if (bytes && !(kernel && std::strcmp(kernel, "popcount") == 0)) {
+      DeviceGuard guard(device);
+      if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes) == hipSuccess) {
+        g->workspace_bytes = bytes;
+      } else {
+        g->workspace = nullptr;
+        (void)hipGetLastError();
+      }
+    }
+  }
   *gemm = g;
   return CCGLIB_OK;
 }
@@ -249,6 +275,8 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   // same switches as the reference's HAVE_ALPHA / HAVE_BETA (src/mma/GEMM.cpp:207-213)
   p.have_alpha = (g->alpha_re != 1.0f || g->alpha_im != 0.0f);
   p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
+  p.workspace = g->workspace;
+  p.workspace_bytes = g->workspace_bytes;
   if (g->K == 0 && g->variant == kOpt) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "K = 0 has no tiled layout");
   }
@@ -261,6 +289,10 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
 }
 
 int ccglib_gemm_destroy(ccglib_gemm_t g) {
+  if (g && g->workspace) {
+    DeviceGuard guard(g->device);
+    (void)hipFree(g->workspace);   // waits for the kernels that still use it
+  }
   delete g;
   return CCGLIB_OK;
 }

@@ -20,6 +20,9 @@ enum ValueType : int {
   kFloat16 = 5,
   kFloat32 = 6
 };
+// Internal operand type of the MFMA path of the 1-bit GEMM: one fp4 (e2m1)
+// value of +1, -1 or 0 per sample. Never crosses the C ABI.
+enum : int { kFp4Sign = 100 };
 enum : int { kPlanar = 0, kInterleaved = 1 };
 enum : int { kForward = 0, kBackward = 1 };
 enum : int { kRowMajor = 0, kColMajor = 1 };
@@ -39,6 +42,7 @@ inline size_t ceil_div(size_t a, size_t b) { return a / b + (a % b != 0); }
 inline int bits_of(int type) {
   switch (type) {
     case kInt1: return 1;
+    case kFp4Sign: return 4;
     case kFloat8e4m3:
     case kFloat8e5m2: return 8;
     case kBfloat16:
@@ -73,7 +77,13 @@ struct GemmParams {
   int c_interleaved;    // 0 planar, 1 interleaved
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta;
+  // 1-bit GEMM only: device memory for the operands expanded to fp4 (may be null)
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
 };
+
+// Bytes of workspace with which the 1-bit GEMM of this size runs in one pass.
+size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k);
 
 hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream);
 hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream);

@@ -175,10 +175,137 @@ hipError_t launch_loader(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// MFMA path. CDNA4 has no 1-bit MFMA, but its fp4 (e2m1) MFMA runs at twice the
+// fp8 rate and +-1 products summed in fp32 are exact integers (up to 2^24), so
+// the packed operands are first expanded - one nibble per sample: 0x2 = +1.0,
+// 0xA = -1.0, 0x0 = 0.0 for the positions past K - into the tiled layout of
+// the MFMA kernel ([batch][rows/128][K/128][2][128 rows][64 bytes]), and the
+// complex GEMM then runs on the matrix cores. With +-1 values the four real
+// products give K - 2 popc(x ^ y) directly, and the zeros make the padding
+// drop out, which is what the reference's K_PADDING correction computes.
+// ---------------------------------------------------------------------------
+typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+
+// 8 bits -> bit i at position 4 i
+__device__ __forceinline__ unsigned spread8(unsigned x) {
+  x = (x | (x << 12)) & 0x000f000fu;
+  x = (x | (x << 6)) & 0x03030303u;
+  x = (x | (x << 3)) & 0x11111111u;
+  return x;
+}
+
+// One thread per 32 samples of one row: one word of bits in, 16 bytes out. A
+// wave reads 4 source rows (256 bytes contiguous) and writes 4 rows x 64 bytes
+// (256 bytes contiguous) into each of four K tiles of the expanded layout.
+// TILED: the source is the 1-bit tiled layout (tiles of 512 samples); otherwise
+// planar rows of k_words words.
+template <bool TILED>
+__global__ __launch_bounds__(256) void expand_int1_to_fp4(const char *__restrict__ src,
+                                                          char *__restrict__ dst, unsigned rows, unsigned row_tiles,
+                                                          unsigned k, unsigned k1_tiles,
+                                                          unsigned k4_tiles, unsigned k_words) {
+  // blockIdx.x: (batch, row tile, source K tile), uniform per block; blockIdx.y
+  // and the thread index: (plane, row, chunk, word) of that tile
+  const unsigned t = blockIdx.y * 256 + threadIdx.x;
+  const unsigned j = t & 3, c = (t >> 2) & 3, row = (t >> 4) & 127, plane = (t >> 11) & 1;
+  const unsigned kt1 = blockIdx.x % k1_tiles;
+  const unsigned rest = blockIdx.x / k1_tiles;
+  const unsigned rt = rest % row_tiles;
+  const size_t b = rest / row_tiles;
+  const unsigned k4 = 4 * kt1 + c;          // K tile of the expanded layout (128 samples)
+  if (k4 >= k4_tiles) return;
+  unsigned bits = 0;
+  if constexpr (TILED) {
+    bits = *reinterpret_cast<const unsigned *>(src + ((b * row_tiles + rt) * k1_tiles + kt1) * kTileBytes +
+                                               plane * kTilePlaneBytes + row * kTileRowBytes + c * 16 +
+                                               j * 4);
+  } else {
+    const unsigned r = rt * kTileRows + row;
+    if (r < rows && 4 * k4 + j < k_words) {
+      bits = reinterpret_cast<const unsigned *>(src)[((b * 2 + plane) * rows + r) * (size_t)k_words +
+                                                     4 * k4 + j];
+    }
+  }
+  // samples of this word that exist: the others become 0.0
+  const unsigned first = k4 * 128 + 32 * j;
+  const unsigned n = first >= k ? 0u : (k - first >= 32 ? 32u : k - first);
+  const unsigned valid = n == 32 ? 0xffffffffu : ((1u << n) - 1u);
+  const unsigned w = bits & valid;
+  uint4_t o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    o[q] = (spread8((w >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
+  }
+  __builtin_nontemporal_store(
+      o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
+                                     plane * kTilePlaneBytes + row * kTileRowBytes + 16 * j));
+}
+
+// Largest K for which every partial sum (at most 2 K in magnitude) is exact in fp32.
+constexpr unsigned kMaxMfmaK = 1u << 22;
+
+hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *done) {
+  *done = false;
+  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
+  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
+  const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
+  const unsigned k_words = (unsigned)ceil_div(p.k, 32);
+  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
+  const size_t y_bytes = (size_t)p.y_tiles * k4_tiles * kTileBytes;
+  const size_t group = p.workspace_bytes / (x_bytes + y_bytes);
+  if (group == 0) return hipSuccess;
+  const bool tiled = (p.variant == kOpt);
+  if (!tiled && (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0)) return hipSuccess;
+  if (tiled && (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0)) return hipSuccess;
+  const size_t x_src = tiled ? (size_t)p.x_tiles * k1_tiles * kTileBytes : (size_t)2 * p.nx * k_words * 4;
+  const size_t y_src = tiled ? (size_t)p.y_tiles * k1_tiles * kTileBytes : (size_t)2 * p.ny * k_words * 4;
+  char *ws_x = static_cast<char *>(p.workspace);
+  for (size_t b0 = 0; b0 < p.batch; b0 += group) {
+    const size_t nb = (p.batch - b0 < group) ? p.batch - b0 : group;
+    char *ws_y = ws_x + nb * x_bytes;
+    for (int which = 0; which < 2; ++which) {
+      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+      const char *src = static_cast<const char *>(which ? p.y : p.x) + b0 * (which ? y_src : x_src);
+      char *dst = which ? ws_y : ws_x;
+      const size_t blocks = nb * row_tiles * k1_tiles;
+      if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+      const dim3 grid((unsigned)blocks, 16);
+      if (tiled) {
+        hipLaunchKernelGGL(expand_int1_to_fp4<true>, grid, dim3(256), 0, stream, src, dst, rows,
+                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
+      } else {
+        hipLaunchKernelGGL(expand_int1_to_fp4<false>, grid, dim3(256), 0, stream, src, dst, rows,
+                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
+      }
+    }
+    GemmParams q = p;
+    q.x = ws_x;
+    q.y = ws_y;
+    q.c = static_cast<char *>(p.c) + b0 * 2 * (size_t)p.nx * p.ny * 4;
+    q.batch = (unsigned)nb;
+    q.k_tiles = k4_tiles;
+    q.type_in = kFp4Sign;
+    q.variant = kOpt;
+    q.input_interleaved = 0;
+    if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
+  }
+  *done = true;
+  return hipGetLastError();
+}
+
 }  // namespace
+
+size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k) {
+  if (k == 0 || k > kMaxMfmaK) return 0;
+  return batch * (ceil_div(m, kTileRows) + ceil_div(n, kTileRows)) * ceil_div(k, 128) * kTileBytes;
+}
 
 hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream) {
   if (p.type_in != kInt1 || p.type_out != kInt32) return hipErrorInvalidValue;
+  bool done = false;
+  if (hipError_t e = launch_int1_on_mfma(p, stream, &done)) return e;
+  if (done) return hipSuccess;
   if (p.variant == kOpt) return launch_loader<kLoadTiled>(p, stream);
   const size_t k_bytes = ceil_div(p.k, 32) * 4;
   const bool aligned = (k_bytes >= 16) && (k_bytes % 16 == 0) && ((uintptr_t)p.x % 16 == 0) &&

@@ -39,8 +39,9 @@ typedef unsigned short ushort4_t __attribute__((ext_vector_type(4)));
 template <int DT> struct DtypeTraits {
   static constexpr int kTilesPerMfma = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 2 : 1;
   static constexpr int kElemBytes = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 1 : 2;
-  static constexpr unsigned kSignMask =
-      (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u : 0x80008000u;
+  static constexpr unsigned kSignMask = (DT == kFp4Sign)                            ? 0x88888888u
+                                        : (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u
+                                                                                   : 0x80008000u;
 };
 
 template <int DT> struct Fragment {
@@ -113,6 +114,16 @@ __device__ __forceinline__ float16_t_ mfma32(const Fragment32 &a, const Fragment
                                                     __builtin_bit_cast(bf16x8_t, b.v[u]), acc, 0, 0, 0);
     }
     return acc;
+  } else if constexpr (DT == kFp4Sign) {
+    // fp4: 64 values of K are 16 bytes per lane, so the 64-byte row is two
+    // instructions (format code 4; only the low four registers are read)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int8_t_ av = {a.v[u][0], a.v[u][1], a.v[u][2], a.v[u][3], 0, 0, 0, 0};
+      const int8_t_ bv = {b.v[u][0], b.v[u][1], b.v[u][2], b.v[u][3], 0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 0, 0x7f, 0, 0x7f);
+    }
+    return acc;
   } else {
     int8_t_ av, bv;
 #pragma unroll
@@ -155,6 +166,7 @@ template <int TOUT> struct OutType;
 template <> struct OutType<kFloat32> { using type = float; };
 template <> struct OutType<kFloat16> { using type = _Float16; };
 template <> struct OutType<kBfloat16> { using type = __bf16; };
+template <> struct OutType<kInt32> { using type = int; };
 
 // One K tile (or two for fp8) of math for a wave: reads its X and Y fragments
 // from the LDS slot(s) and issues the four real products of the complex MAC.
@@ -408,6 +420,85 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
   }
 }
 
+// Epilogue of the 1-bit GEMM on the MFMA path: the accumulators hold exact
+// integers (sums of +-1 products); alpha and beta are truncated to integers and
+// everything wraps modulo 2^32, as in the popcount kernel.
+template <int TX, int TY, int MS, typename Acc>
+__device__ __forceinline__ void store_wave_tile_int32(const KernelArgs &args, unsigned b,
+                                                      unsigned x_wave, unsigned y_wave, int lane,
+                                                      const Acc &acc_re, const Acc &acc_im) {
+  constexpr int NPX = MS == 16 ? TX : TX * 4;
+  const unsigned nx = args.nx, ny = args.ny;
+  const unsigned ar = (unsigned)(int)args.alpha_re, ai = (unsigned)(int)args.alpha_im;
+  const unsigned br = (unsigned)(int)args.beta_re, bi = (unsigned)(int)args.beta_im;
+  const bool have_beta = args.have_beta;
+  unsigned *cbase = reinterpret_cast<unsigned *>(args.c) + (size_t)b * 2 * nx * ny;
+  const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+    const unsigned y = y_wave + piece_y<MS>(j, lane);
+#pragma unroll
+    for (int i = 0; i < NPX; ++i) {
+      const unsigned x = x_wave + piece_x<MS>(i, lane);
+      if (y >= ny || x >= nx) continue;
+      unsigned re[4], im[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const unsigned sr = (unsigned)(int)piece_elem<MS>(acc_re, j, i, e);
+        const unsigned si = (unsigned)(int)piece_elem<MS>(acc_im, j, i, e);
+        re[e] = ar * sr - ai * si;
+        im[e] = ai * sr + ar * si;
+      }
+      const bool full = vec_ok && (x + 4 <= nx);
+      if (!args.c_interleaved) {
+        unsigned *pr = cbase + (size_t)y * nx + x, *pi = pr + (size_t)nx * ny;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (have_beta && x + e < nx) {
+            const unsigned cr = pr[e], ci = pi[e];
+            re[e] += br * cr - bi * ci;
+            im[e] += bi * cr + br * ci;
+          }
+        }
+        if (full) {
+          *reinterpret_cast<int4_t *>(pr) = int4_t{(int)re[0], (int)re[1], (int)re[2], (int)re[3]};
+          *reinterpret_cast<int4_t *>(pi) = int4_t{(int)im[0], (int)im[1], (int)im[2], (int)im[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              pr[e] = re[e];
+              pi[e] = im[e];
+            }
+          }
+        }
+      } else {
+        unsigned *p = cbase + ((size_t)y * nx + x) * 2;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (have_beta && x + e < nx) {
+            const unsigned cr = p[2 * e], ci = p[2 * e + 1];
+            re[e] += br * cr - bi * ci;
+            im[e] += bi * cr + br * ci;
+          }
+        }
+        if (full) {
+          reinterpret_cast<int4_t *>(p)[0] = int4_t{(int)re[0], (int)im[0], (int)re[1], (int)im[1]};
+          reinterpret_cast<int4_t *>(p)[1] = int4_t{(int)re[2], (int)im[2], (int)re[3], (int)im[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (x + e < nx) {
+              p[2 * e] = re[e];
+              p[2 * e + 1] = im[e];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 // Epilogue through LDS for the common case (planar fp32 C, beta = 0, wave tile
 // entirely inside C, 64 columns wide): the accumulators of 16 rows are written
 // to a wave-private LDS patch and read back row-wise, so that every store
@@ -458,7 +549,7 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
 // instruction writes eight whole 128-byte row segments.
 constexpr int kStagePatch32Bytes = 32 * 144;
 
-template <int TX, int TY>
+template <int TX, int TY, bool INT = false>
 __device__ __forceinline__ void store_wave_tile_staged32(const KernelArgs &args, unsigned b,
                                                          unsigned x_wave, unsigned y_wave, int lane,
                                                          char *patch, float16_t_ (&acc_re)[TY][TX],
@@ -482,8 +573,16 @@ __device__ __forceinline__ void store_wave_tile_staged32(const KernelArgs &args,
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float re = acc_re[j][i][4 * k + e], im = acc_im[j][i][4 * k + e];
-            v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
-                              : (have_alpha ? ai * re + ar * im : im);
+            if constexpr (INT) {
+              // exact integers; alpha truncated, arithmetic modulo 2^32
+              const unsigned sr = (unsigned)(int)re, si = (unsigned)(int)im;
+              const unsigned iar = (unsigned)(int)ar, iai = (unsigned)(int)ai;
+              const unsigned o = plane == 0 ? iar * sr - iai * si : iai * sr + iar * si;
+              v[e] = __builtin_bit_cast(float, o);
+            } else {
+              v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
+                                : (have_alpha ? ai * re + ar * im : im);
+            }
           }
           *reinterpret_cast<float4_t *>(wr + k * 32) = v;
         }
@@ -889,13 +988,14 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         }
       }
     }
-    if constexpr (MS == 32 && TOUT == kFloat32 && NW * kStagePatch32Bytes <= KPI * SLOT_BYTES) {
+    if constexpr (MS == 32 && (TOUT == kFloat32 || TOUT == kInt32) &&
+                  NW * kStagePatch32Bytes <= KPI * SLOT_BYTES) {
       if (staged_ok) {
         unsigned free_slot = slot + LEAD * KPI;
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
-          store_wave_tile_staged32<TX, TY>(args, tc.b, x_wave, y_wave, lane,
+          store_wave_tile_staged32<TX, TY, TOUT == kInt32>(args, tc.b, x_wave, y_wave, lane,
                                            lds + free_slot * SLOT_BYTES + wave * kStagePatch32Bytes,
                                            acc_re, acc_im);
           staged = true;
@@ -903,7 +1003,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     if (!staged) {
-      store_wave_tile<TOUT, TX, TY, MS>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+      if constexpr (TOUT == kInt32) {
+        store_wave_tile_int32<TX, TY, MS>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+      } else {
+        store_wave_tile<TOUT, TX, TY, MS>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+      }
     }
   }
   // nothing may still be writing into LDS when the block gives it back
@@ -1029,6 +1133,12 @@ hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
       break;
     case kFloat8e5m2:
       if (p.type_out == kFloat32) return launch_typed<kFloat8e5m2, kFloat32>(p, stream);
+      break;
+    case kFp4Sign:
+      // the 1-bit GEMM's operands expanded to fp4 +-1, tiled; exact integer sums
+      if (p.type_out == kInt32 && p.variant == kOpt && !p.input_interleaved) {
+        return launch_dtl<kFp4Sign, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream);
+      }
       break;
     default:
       break;
