@@ -184,6 +184,9 @@ hipError_t launch_loader(const GemmParams &p, hipStream_t stream) {
 // complex GEMM then runs on the matrix cores. With +-1 values the four real
 // products give K - 2 popc(x ^ y) directly, and the zeros make the padding
 // drop out, which is what the reference's K_PADDING correction computes.
+// (Bits past K inside the last word are ignored here; the popcount kernel and
+// the reference count them and so require them to be zero, which Packing
+// guarantees. For such input both paths give the same result.)
 // ---------------------------------------------------------------------------
 typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
 

@@ -209,6 +209,22 @@ def test_batches_are_independent():
 
 # ---- 1-bit ------------------------------------------------------------------------------
 
+@pytest.fixture(params=["mfma", "mfma_grouped", "popcount"])
+def int1_kernel(request, monkeypatch):
+    """The 1-bit GEMM has two implementations behind one entry point: fp4 MFMA on
+    expanded operands (default; "grouped" = a workspace cap that forces several
+    passes over groups of batches) and XOR + popcount on the vector ALUs (used
+    when K is too large for exact fp32 sums or the workspace cannot be had). The
+    choice is read from the environment when the GEMM object is created."""
+    monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
+    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
+    if request.param == "popcount":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
+    elif request.param == "mfma_grouped":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+    return request.param
+
+
 def int1_case(B, M, N, K, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0, seed=0):
     rng = np.random.default_rng(seed)
     kw = (K + 31) // 32
@@ -252,21 +268,47 @@ def test_kat_int1():
 @pytest.mark.parametrize("c_order", [ROW, COL])
 @pytest.mark.parametrize("M,N,K", [(64, 64, 256), (128, 128, 512), (100, 60, 1024), (130, 257, 96),
                                    (256, 128, 4096)])
-def test_int1(variant, c_order, M, N, K):
+def test_int1(variant, c_order, M, N, K, int1_kernel):
     int1_case(16 if M == 64 else 3, M, N, K, variant, PLANAR, c_order, seed=M)
 
 
 @pytest.mark.parametrize("c_order", [ROW, COL])
-def test_int1_interleaved_output(c_order):
+def test_int1_interleaved_output(c_order, int1_kernel):
     int1_case(2, 100, 60, 512, cc.Variant.opt, INTERLEAVED, c_order)
 
 
-@pytest.mark.parametrize("K", [45, 100])
-def test_int1_k_not_multiple_of_32(K):
+@pytest.mark.parametrize("K", [45, 100, 1000])
+def test_int1_k_not_multiple_of_32(K, int1_kernel):
     int1_case(2, 20, 30, K, cc.Variant.basic, seed=K)
 
 
+@pytest.mark.parametrize("K", [32, 160, 1056])
+def test_int1_k_not_multiple_of_a_tile(K, int1_kernel):
+    # whole words, but neither whole 128-sample nor whole 512-sample tiles
+    int1_case(2, 130, 70, K, cc.Variant.opt, seed=K + 1)
+    int1_case(2, 130, 70, K, cc.Variant.basic, seed=K + 2)
+
+
+def test_int1_largest_k_of_the_mfma_path_and_beyond():
+    # K = 2^22 is the largest the fp4 path takes (sums up to 2 K = 2^23 stay exact in
+    # fp32); identical operands give the extreme value im = 2 K in every element.
+    # One tile more and the popcount kernel takes over.
+    for K in (1 << 22, (1 << 22) + 512):
+        kw = K // 32
+        rng = np.random.default_rng(K)
+        row = rng.integers(0, 2 ** 32, kw, dtype=np.uint32)
+        a = np.broadcast_to(row, (1, 2, 8, kw)).copy().reshape(-1)
+        b = np.broadcast_to(row, (1, 2, 4, kw)).copy().reshape(-1)
+        d_a, d_b = transpose_operand(a, 1, 8, K, VT.int1), transpose_operand(b, 1, 4, K, VT.int1)
+        d_c = to_device(np.zeros(2 * 8 * 4, np.int32))
+        cc.GEMM(1, 8, 4, K, 0, stream(), cc.Precision(VT.int1, VT.int32), cc.Variant.opt).Run(
+            d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+        torch.cuda.synchronize()
+        got = to_host(d_c, np.int32).reshape(2, 8, 4)
+        assert (got[0] == 0).all() and (got[1] == 2 * K).all()
+
+
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
-def test_int1_alpha_beta(variant):
+def test_int1_alpha_beta(variant, int1_kernel):
     # test/gemm/mma.cpp:713-775
     int1_case(16, 256, 128, 256, variant, alpha=2 - 3j, beta=3 - 2j)
