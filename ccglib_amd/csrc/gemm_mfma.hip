@@ -171,10 +171,11 @@ template <> struct OutType<kInt32> { using type = int; };
 // One K tile (or two for fp8) of math for a wave: reads its X and Y fragments
 // from the LDS slot(s) and issues the four real products of the complex MAC.
 // slot[u] points at the K tile u of this MFMA step: [X re][X im][Y re][Y im].
-template <int DT, int BX, int BY, int TX, int TY>
+template <int DT, int BX, int BY, int TX, int TY, typename Mid>
 __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<DT>::kTilesPerMfma],
                                          int x_frag_off, int y_frag_off,
-                                         float4_t (&acc_re)[TY][TX], float4_t (&acc_im)[TY][TX]) {
+                                         float4_t (&acc_re)[TY][TX], float4_t (&acc_im)[TY][TX],
+                                         Mid &&mid) {
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
   Fragment<DT> xr[TX], xi[TX];
 #pragma unroll
@@ -204,15 +205,16 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
     for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
 #pragma unroll
     for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
+    if (j == 0) mid();
   }
 }
 
 // The same on the 32-row MFMAs: TX x TY tiles of 32x32, one K tile per step.
 // off[0] and off[1] are the lane's two 16-byte chunks of its row.
-template <int DT, int BX, int BY, int TX, int TY>
+template <int DT, int BX, int BY, int TX, int TY, typename Mid>
 __device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[2],
                                            const int (&y_off)[2], float16_t_ (&acc_re)[TY][TX],
-                                           float16_t_ (&acc_im)[TY][TX]) {
+                                           float16_t_ (&acc_im)[TY][TX], Mid &&mid) {
   constexpr int D = TX > TY ? TX : TY;
   Fragment32 xr[TX], xi[TX], yr[TY], yi[TY], yin[TY];
 #pragma unroll
@@ -265,6 +267,10 @@ __device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[
 #pragma unroll
     for (int t = 0; t < n; ++t)
       acc_im[tj[t]][ti[t]] = mfma32<DT>(xi[ti[t]], yr[tj[t]], acc_im[tj[t]][ti[t]]);
+    if (d == 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      mid();
+    }
   }
   __builtin_amdgcn_sched_barrier(0);
 }
@@ -276,11 +282,11 @@ __device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[
 // Y fragment in registers: a sign flip of the odd elements and a swap inside
 // each pair. Two MFMAs per fragment pair over half as many complex values:
 // the same MFMA and LDS work per complex MAC as with planar operands.
-template <int DT, int BX, int BY, int TX, int TY>
+template <int DT, int BX, int BY, int TX, int TY, typename Mid>
 __device__ __forceinline__ void mma_step_interleaved(const char *slot, const int (&x_off)[2],
                                                      const int (&y_off)[2],
                                                      float4_t (&acc_re)[TY][TX],
-                                                     float4_t (&acc_im)[TY][TX]) {
+                                                     float4_t (&acc_im)[TY][TX], Mid &&mid) {
   // The slot holds 128 bytes of every row; x_off / y_off are the lane's two
   // 16-byte chunks of its row. fp8 takes both in one MFMA, 16-bit input one
   // per MFMA (two passes over the slot).
@@ -316,6 +322,7 @@ __device__ __forceinline__ void mma_step_interleaved(const char *slot, const int
       for (int i = 0; i < TX; ++i) acc_re[j][i] = mfma<DT>(x[i], y1, acc_re[j][i]);
 #pragma unroll
       for (int i = 0; i < TX; ++i) acc_im[j][i] = mfma<DT>(x[i], y2, acc_im[j][i]);
+      if (h == 0 && j == 0) mid();
     }
   }
 }
@@ -694,7 +701,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       const char *slot[KPM];
 #pragma unroll
       for (int u = 0; u < KPM; ++u) slot[u] = s + (kk + u) * KTILE_BYTES;
-      mma_step<DT, BX, BY, TX, TY>(slot, x_frag_off, y_frag_off, acc_re, acc_im);
+      mma_step<DT, BX, BY, TX, TY>(slot, x_frag_off, y_frag_off, acc_re, acc_im, [] {});
     }
   };
 
@@ -867,8 +874,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     }
   };
   auto issue_next = [&](int slot) {
-    const bool real = (load_tile < total) && (load_kt < k_tiles);
+    // Past the last C tile the copy re-reads the last one (never used); only K
+    // tiles past the end of K, whose contents enter the sums, read zeros.
     if constexpr (LOADER == kLoadTiled) {
+      const bool real = (KPI == 1) || (load_kt < k_tiles);
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
         const char *base = real ? src[i] + (size_t)load_kt * kTileBytes + tile_off[i] : g_zero_tile;
@@ -876,7 +885,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
-      const bool inside = real && (load_kt * RB + c * 16 + 16 <= row_bytes);
+      const bool inside = (load_kt * RB + c * 16 + 16 <= row_bytes);
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
         const char *p = inside ? lane_src[i] + (size_t)load_kt * RB
@@ -944,19 +953,24 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       // K tiles that are LEAD iterations ahead (of this C tile or the next)
       unsigned refill = slot + LEAD * KPI;
       refill = refill >= SLOTS ? refill - SLOTS : refill;
+      // The copy instructions go out after the first group of MFMAs: right
+      // after the barrier every wave of the block would otherwise be busy with
+      // their address arithmetic and the matrix cores would have nothing to do.
+      auto refill_slots = [&] {
 #pragma unroll
-      for (int u = 0; u < KPI; ++u) issue_next(refill + u);
+        for (int u = 0; u < KPI; ++u) issue_next(refill + u);
+      };
       if constexpr (IL) {
         mma_step_interleaved<DT, BX, BY, TX, TY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
-                                                 acc_im);
+                                                 acc_im, refill_slots);
       } else {
         const char *tile[KPM];
 #pragma unroll
         for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
         if constexpr (MS == 32) {
-          mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im);
+          mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
         } else {
-          mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im);
+          mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
         }
       }
       slot += KPI;
