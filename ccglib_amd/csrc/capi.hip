@@ -83,6 +83,7 @@ bool pair_supported(int in, int out) {
   switch (in) {
     case kFloat16: return out == kFloat32 || out == kFloat16;
     case kBfloat16: return out == kFloat32 || out == kBfloat16;
+    case kFloat32: return out == kFloat32 || out == kFloat16 || out == kBfloat16;
     case kFloat8e4m3:
     case kFloat8e5m2: return out == kFloat32;
     case kInt1: return out == kInt32;

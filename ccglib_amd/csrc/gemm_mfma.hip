@@ -38,9 +38,12 @@ typedef unsigned short ushort4_t __attribute__((ext_vector_type(4)));
 // (16x16x128: 32 bytes per lane, 16 from each of two K tiles).
 template <int DT> struct DtypeTraits {
   static constexpr int kTilesPerMfma = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 2 : 1;
-  static constexpr int kElemBytes = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 1 : 2;
+  static constexpr int kElemBytes = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 1
+                                    : (DT == kFloat32)                       ? 4
+                                                                             : 2;
   static constexpr unsigned kSignMask = (DT == kFp4Sign)                            ? 0x88888888u
                                         : (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u
+                                        : (DT == kFloat32)                         ? 0x80000000u
                                                                                    : 0x80008000u;
 };
 
@@ -57,6 +60,19 @@ __device__ __forceinline__ float4_t mfma(const Fragment<DT> &a, const Fragment<D
   } else if constexpr (DT == kBfloat16) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
         __builtin_bit_cast(bf16x8_t, a.v[0]), __builtin_bit_cast(bf16x8_t, b.v[0]), acc, 0, 0, 0);
+  } else if constexpr (DT == kFloat32) {
+    // fp32 input (true fp32 products, no tf32 on this part): a lane's 16-byte
+    // chunk is four K values; 16x16x4 takes one value per lane, and which K a
+    // lane supplies does not matter as long as both operands agree.
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // (copies first: a bit cast applied to a vector element expression
+      // directly reads element 0 whatever the index)
+      const int ae = a.v[0][e], be = b.v[0][e];
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, ae),
+                                                 __builtin_bit_cast(float, be), acc, 0, 0, 0);
+    }
+    return acc;
   } else {
     int8_t_ av, bv;
 #pragma unroll
@@ -1103,8 +1119,10 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
                              ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.y % 16 == 0);
   if (p.input_interleaved) {
     // raw (re, im) rows straight from the caller: the host side only takes this
-    // path when the rows are whole aligned 16-byte chunks
-    if constexpr (KPM == 1) {
+    // path for 8- and 16-bit input whose rows are whole aligned 16-byte chunks
+    if constexpr (DT == kFloat32) {
+      return hipErrorInvalidValue;
+    } else if constexpr (KPM == 1) {
       return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec>(p, stream);
     } else {
       return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec>(p, stream);
@@ -1112,7 +1130,7 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   }
   if (p.variant == kOpt || planar_direct) {
     if constexpr (KPM == 1) {
-      // 16-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
+      // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
       return p.variant == kOpt
                  ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled>(p, stream)
                  : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec>(p, stream);
@@ -1141,6 +1159,11 @@ hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
     case kBfloat16:
       if (p.type_out == kFloat32) return launch_typed<kBfloat16, kFloat32>(p, stream);
       if (p.type_out == kBfloat16) return launch_typed<kBfloat16, kBfloat16>(p, stream);
+      break;
+    case kFloat32:
+      if (p.type_out == kFloat32) return launch_typed<kFloat32, kFloat32>(p, stream);
+      if (p.type_out == kFloat16) return launch_typed<kFloat32, kFloat16>(p, stream);
+      if (p.type_out == kBfloat16) return launch_typed<kFloat32, kBfloat16>(p, stream);
       break;
     case kFloat8e4m3:
       if (p.type_out == kFloat32) return launch_typed<kFloat8e4m3, kFloat32>(p, stream);

@@ -79,8 +79,10 @@ CCGLIB_API const char *ccglib_version(void);
  *   C:     planar [B][2][M][N] (row major) / [B][2][N][M] (column major);
  *          interleaved [B][M][N][2] / [B][N][M][2] (opt variant only)
  * Supported (type_in -> type_out): float16->float32|float16,
- * bfloat16->float32|bfloat16, float8e4m3->float32, float8e5m2->float32,
- * int1->int32. Accumulation is float32 (int32 for 1-bit input).
+ * bfloat16->float32|bfloat16, float32->float32|float16|bfloat16,
+ * float8e4m3->float32, float8e5m2->float32, int1->int32 (the reference's
+ * matrix, kernels/type_selector.h:65-212). Accumulation is float32 (int32 for
+ * 1-bit input).
  * a_order must be row major and b_order column major (as in the reference,
  * where anything else fails to compile: kernels/gemm_kernel_float.cu:20-25);
  * the error text keeps the token HIPRTC_ERROR_COMPILATION that the

@@ -13,16 +13,22 @@ ORC_TYPE = {cc.ValueType.float16: orc.FLOAT16, cc.ValueType.bfloat16: orc.BFLOAT
 
 # per-element tolerance of the reference's own tests (test/gemm/fpequals.h:15-53)
 EPSILON = {cc.ValueType.float8e4m3: 0.125, cc.ValueType.float8e5m2: 0.25,
-           cc.ValueType.float16: 0.000976562, cc.ValueType.bfloat16: 0.0078125}
+           cc.ValueType.float16: 0.000976562, cc.ValueType.bfloat16: 0.0078125,
+           # the reference runs float32 input as tf32 and tests it with the fp16 epsilon; the
+           # products here are true fp32, so the Frobenius bound below is the tight one
+           cc.ValueType.float32: 0.000976562}
 # relative Frobenius error bound against float64
 FROBENIUS = {cc.ValueType.float16: 1e-3, cc.ValueType.bfloat16: 1e-3,
-             cc.ValueType.float8e4m3: 2e-2, cc.ValueType.float8e5m2: 2e-2}
+             cc.ValueType.float8e4m3: 2e-2, cc.ValueType.float8e5m2: 2e-2,
+             cc.ValueType.float32: 1e-5}
 
 
 def quantize(x, vtype):
     """float32 array -> storage bit patterns (round to nearest even, fp8 saturating)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     t = torch.from_numpy(x)
+    if vtype == cc.ValueType.float32:
+        return x
     if vtype == cc.ValueType.float16:
         return x.astype(np.float16).view(np.uint16)
     if vtype == cc.ValueType.bfloat16:

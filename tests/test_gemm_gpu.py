@@ -18,7 +18,8 @@ ROW, COL = cc.MemOrder.row_major, cc.MemOrder.col_major
 OUT_NP = {VT.float32: np.float32, VT.float16: np.uint16, VT.bfloat16: np.uint16, VT.int32: np.int32}
 
 FLOAT_PAIRS = [(VT.float16, VT.float32), (VT.float16, VT.float16), (VT.bfloat16, VT.float32),
-               (VT.bfloat16, VT.bfloat16), (VT.float8e4m3, VT.float32), (VT.float8e5m2, VT.float32)]
+               (VT.bfloat16, VT.bfloat16), (VT.float8e4m3, VT.float32), (VT.float8e5m2, VT.float32),
+               (VT.float32, VT.float32), (VT.float32, VT.float16), (VT.float32, VT.bfloat16)]
 
 
 def run_gemm(qa, qb, B, M, N, K, tin, tout, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0,
@@ -88,7 +89,7 @@ KAT_A = [1, 2, 3, 4, 5, 6, 6, 5, 4, 3, 2, 1]
 KAT_B = [1, 2, 3, 4, 4, 3, 2, 1]
 
 
-@pytest.mark.parametrize("tin", [VT.float16, VT.bfloat16])
+@pytest.mark.parametrize("tin", [VT.float16, VT.bfloat16, VT.float32])
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
 def test_kat_float(tin, variant):
     qa, qb = quantize(np.array(KAT_A), tin), quantize(np.array(KAT_B), tin)
@@ -142,6 +143,19 @@ def test_opt(tin, tout, M, N, K, c_order, c_axis):
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
 def test_odd_shapes_fp16(M, N, K, variant):
     float_case(2, M, N, K, VT.float16, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000), (257, 129, 72)])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_odd_shapes_fp32(M, N, K, variant):
+    # K not a multiple of the 16 values of a tile row, rows that are not whole 16-byte chunks
+    float_case(2, M, N, K, VT.float32, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
+
+
+def test_fp32_alpha_beta_and_many_tiles():
+    float_case(3, 256, 320, 96, VT.float32, VT.float32, cc.Variant.opt, INTERLEAVED, COL,
+               alpha=0.75 - 0.5j, beta=0.5 - 0.25j)
+    float_case(40, 256, 1024, 32, VT.float32, VT.float16, cc.Variant.opt, PLANAR, ROW, seed=13)
 
 
 @pytest.mark.parametrize("tin", [VT.float8e4m3, VT.float8e5m2])

@@ -6,7 +6,7 @@ import torch
 
 import ccglib_amd as cc
 import oracle as orc
-from gpu_util import ORC_TYPE, check_float, quantize, stream, to_device, to_host
+from gpu_util import ORC_TYPE, check_float, dequantize, quantize, stream, to_device, to_host
 
 pytestmark = pytest.mark.gpu
 VT = cc.ValueType
@@ -59,6 +59,26 @@ def test_pipeline_interleaved_in_and_out():
     want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, orc.BFLOAT16, orc.FLOAT32, orc.COL_MAJOR)
     w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, orc.BFLOAT16, orc.COL_MAJOR)
     check_float(got, want, w64, VT.bfloat16, VT.float32)
+
+
+def test_pipeline_fp32_interleaved_in():
+    # 32-bit interleaved input is not consumed directly: it goes through the transposes
+    B, M, N, K = 2, 130, 70, 50
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32)
+    a_il = np.ascontiguousarray(a.transpose(0, 2, 3, 1))
+    b_il = np.ascontiguousarray(b.transpose(0, 2, 3, 1))
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, VT.float32,
+                    VT.float16, cc.Variant.opt)
+    d_a, d_b = to_device(a_il.reshape(-1)), to_device(b_il.reshape(-1))
+    d_c = to_device(np.full(B * 2 * M * N, 0x7fc0, dtype=np.uint16))
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = dequantize(to_host(d_c, np.uint16), VT.float16).reshape(B, 2, M, N)
+    want = orc.gemm(a.reshape(-1), b.reshape(-1), M, N, K, orc.FLOAT32, orc.FLOAT16)
+    w64 = orc.gemm_float64(a.reshape(-1), b.reshape(-1), M, N, K, orc.FLOAT32)
+    check_float(got, dequantize(want, VT.float16), w64, VT.float32, VT.float16)
 
 
 @pytest.mark.parametrize("variant", [cc.Variant.opt, cc.Variant.basic])
