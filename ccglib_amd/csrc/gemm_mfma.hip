@@ -225,6 +225,90 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
   }
 }
 
+// The same step with every LDS read placed by hand, for one K tile per MFMA and
+// a 4 x 4 wave tile. Right after the barrier all waves of the block want their
+// fragments at once and the LDS serves them one read at a time; if a wave asks
+// for all ten fragments of the first tile row before its first MFMA, the matrix
+// cores wait for the whole queue. Here a wave reads what its first MFMA needs,
+// keeps about three reads in flight ahead of their use, and fetches the Y
+// fragments of the next tile row during the current one.
+template <int DT, int BX, int BY, typename Mid>
+__device__ __forceinline__ void mma_step_ordered(const char *slot, int x_frag_off, int y_frag_off,
+                                                 float4_t (&acc_re)[4][4], float4_t (&acc_im)[4][4],
+                                                 Mid &&mid) {
+  static_assert(DtypeTraits<DT>::kTilesPerMfma == 1, "one K tile per MFMA");
+  auto rd = [&](int off) {
+    Fragment<DT> f;
+    f.v[0] = *reinterpret_cast<const int4_t *>(slot + off);
+    return f;
+  };
+  constexpr int ROW16 = 16 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+  Fragment<DT> xr[4], xi[4], yr, yi, yin, yr_next, yi_next;
+  yr = rd(y_frag_off);
+  xr[0] = rd(x_frag_off);
+  xr[1] = rd(x_frag_off + ROW16);
+  xr[2] = rd(x_frag_off + 2 * ROW16);
+  CCGLIB_PIN;
+  acc_re[0][0] = mfma<DT>(xr[0], yr, acc_re[0][0]);
+  xr[3] = rd(x_frag_off + 3 * ROW16);
+  CCGLIB_PIN;
+  acc_re[0][1] = mfma<DT>(xr[1], yr, acc_re[0][1]);
+  yi = rd(y_frag_off + YP);
+  CCGLIB_PIN;
+  acc_re[0][2] = mfma<DT>(xr[2], yr, acc_re[0][2]);
+  xi[0] = rd(x_frag_off + XP);
+  CCGLIB_PIN;
+  acc_re[0][3] = mfma<DT>(xr[3], yr, acc_re[0][3]);
+  xi[1] = rd(x_frag_off + XP + ROW16);
+  CCGLIB_PIN;
+  acc_im[0][0] = mfma<DT>(xr[0], yi, acc_im[0][0]);
+  xi[2] = rd(x_frag_off + XP + 2 * ROW16);
+  CCGLIB_PIN;
+  acc_im[0][1] = mfma<DT>(xr[1], yi, acc_im[0][1]);
+  xi[3] = rd(x_frag_off + XP + 3 * ROW16);
+  CCGLIB_PIN;
+  acc_im[0][2] = mfma<DT>(xr[2], yi, acc_im[0][2]);
+  yin = negate<DT>(yi);
+  CCGLIB_PIN;
+  acc_im[0][3] = mfma<DT>(xr[3], yi, acc_im[0][3]);
+  yr_next = rd(y_frag_off + ROW16);
+  CCGLIB_PIN;
+  acc_re[0][0] = mfma<DT>(xi[0], yin, acc_re[0][0]);
+  yi_next = rd(y_frag_off + YP + ROW16);
+  CCGLIB_PIN;
+  acc_im[0][0] = mfma<DT>(xi[0], yr, acc_im[0][0]);
+#pragma unroll
+  for (int i = 1; i < 4; ++i) {
+    acc_re[0][i] = mfma<DT>(xi[i], yin, acc_re[0][i]);
+    acc_im[0][i] = mfma<DT>(xi[i], yr, acc_im[0][i]);
+  }
+  CCGLIB_PIN;
+  mid();
+  CCGLIB_PIN;
+#pragma unroll
+  for (int j = 1; j < 4; ++j) {
+    yr = yr_next;
+    yi = yi_next;
+    yin = negate<DT>(yi);
+    CCGLIB_PIN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_re[j][i] = mfma<DT>(xr[i], yr, acc_re[j][i]);
+    if (j < 3) yr_next = rd(y_frag_off + (j + 1) * ROW16);
+    CCGLIB_PIN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_im[j][i] = mfma<DT>(xr[i], yi, acc_im[j][i]);
+    if (j < 3) yi_next = rd(y_frag_off + YP + (j + 1) * ROW16);
+    CCGLIB_PIN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
+    CCGLIB_PIN;
+  }
+#undef CCGLIB_PIN
+}
+
 // The same on the 32-row MFMAs: TX x TY tiles of 32x32, one K tile per step.
 // off[0] and off[1] are the lane's two 16-byte chunks of its row.
 template <int DT, int BX, int BY, int TX, int TY, typename Mid>
@@ -985,6 +1069,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
         if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+        } else if constexpr (KPM == 1 && TX == 4 && TY == 4) {
+          mma_step_ordered<DT, BX, BY>(tile[0], x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
         } else {
           mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
         }
