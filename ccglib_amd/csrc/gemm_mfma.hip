@@ -375,6 +375,71 @@ __device__ __forceinline__ void mma_step32(const char *slot, const int (&x_off)[
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// The 32-row step for a 2 x 2 wave tile with the LDS reads in order of need
+// (see mma_step_ordered): two 16-byte reads per fragment.
+template <int DT, int BX, int BY, typename Mid>
+__device__ __forceinline__ void mma_step32_ordered(const char *slot, const int (&x_off)[2],
+                                                   const int (&y_off)[2], float16_t_ (&acc_re)[2][2],
+                                                   float16_t_ (&acc_im)[2][2], Mid &&mid) {
+  auto rd = [&](const int (&off)[2], int extra) {
+    Fragment32 f;
+    f.v[0] = *reinterpret_cast<const int4_t *>(slot + off[0] + extra);
+    f.v[1] = *reinterpret_cast<const int4_t *>(slot + off[1] + extra);
+    return f;
+  };
+  auto neg = [](const Fragment32 &f) {
+    Fragment32 r;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) r.v[u][w] = f.v[u][w] ^ (int)DtypeTraits<DT>::kSignMask;
+    }
+    return r;
+  };
+  constexpr int ROW32 = 32 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+  Fragment32 x0r, x0i, x1r, x1i, y0r, y0i, y0n, y1r, y1i, y1n;
+  y0r = rd(y_off, 0);
+  x0r = rd(x_off, 0);
+  y0i = rd(y_off, YP);
+  CCGLIB_PIN;
+  acc_re[0][0] = mfma32<DT>(x0r, y0r, acc_re[0][0]);
+  x0i = rd(x_off, XP);
+  CCGLIB_PIN;
+  acc_im[0][0] = mfma32<DT>(x0r, y0i, acc_im[0][0]);
+  y0n = neg(y0i);
+  x1r = rd(x_off, ROW32);
+  CCGLIB_PIN;
+  acc_re[0][0] = mfma32<DT>(x0i, y0n, acc_re[0][0]);
+  x1i = rd(x_off, XP + ROW32);
+  CCGLIB_PIN;
+  acc_im[0][0] = mfma32<DT>(x0i, y0r, acc_im[0][0]);
+  CCGLIB_PIN;
+  mid();
+  CCGLIB_PIN;
+  acc_re[0][1] = mfma32<DT>(x1r, y0r, acc_re[0][1]);
+  y1r = rd(y_off, ROW32);
+  CCGLIB_PIN;
+  acc_im[0][1] = mfma32<DT>(x1r, y0i, acc_im[0][1]);
+  y1i = rd(y_off, YP + ROW32);
+  CCGLIB_PIN;
+  acc_re[0][1] = mfma32<DT>(x1i, y0n, acc_re[0][1]);
+  acc_im[0][1] = mfma32<DT>(x1i, y0r, acc_im[0][1]);
+  CCGLIB_PIN;
+  acc_re[1][0] = mfma32<DT>(x0r, y1r, acc_re[1][0]);
+  acc_im[1][0] = mfma32<DT>(x0r, y1i, acc_im[1][0]);
+  y1n = neg(y1i);
+  CCGLIB_PIN;
+  acc_re[1][0] = mfma32<DT>(x0i, y1n, acc_re[1][0]);
+  acc_im[1][0] = mfma32<DT>(x0i, y1r, acc_im[1][0]);
+  acc_re[1][1] = mfma32<DT>(x1r, y1r, acc_re[1][1]);
+  acc_im[1][1] = mfma32<DT>(x1r, y1i, acc_im[1][1]);
+  acc_re[1][1] = mfma32<DT>(x1i, y1n, acc_re[1][1]);
+  acc_im[1][1] = mfma32<DT>(x1i, y1r, acc_im[1][1]);
+  CCGLIB_PIN;
+#undef CCGLIB_PIN
+}
+
 // The same for interleaved operands (rows of (re, im) pairs, as the caller's
 // buffers hold them). With K running over the 2K real numbers of a row,
 //   Re = sum X~ . Y1,  Y1 = (yr, -yi, ...)   and   Im = sum X~ . Y2,  Y2 = (yi, yr, ...)
@@ -973,7 +1038,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
   };
-  auto issue_next = [&](int slot) {
+  // issue_copies: straight-line code (it is placed between MFMAs, and a
+  // branch there would let the compiler sink those MFMAs below it);
+  // advance_copy: the bookkeeping, with the branches of the tile change.
+  auto issue_copies = [&](int slot) {
     // Past the last C tile the copy re-reads the last one (never used); only K
     // tiles past the end of K, whose contents enter the sums, read zeros.
     if constexpr (LOADER == kLoadTiled) {
@@ -993,11 +1061,17 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
       }
     }
+  };
+  auto advance_copy = [&] {
     if (++load_kt == k_tiles_padded) {
       load_kt = 0;
       load_tile += gridDim.x;
       point_at(load_tile);
     }
+  };
+  auto issue_next = [&](int slot) {
+    issue_copies(slot);
+    advance_copy();
   };
 
   const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
@@ -1025,8 +1099,18 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
 
   // ---- pipeline ----------------------------------------------------------
   point_at(load_tile);
+  // With one slot per iteration the bookkeeping of the copy (advance_copy, which
+  // branches) is done at the top of an iteration for the copies issued inside it,
+  // so that nothing but straight-line code follows the barrier.
 #pragma unroll
-  for (int t = 0; t < LEAD * KPI; ++t) issue_next(t);
+  for (int t = 0; t < LEAD * KPI; ++t) {
+    if constexpr (KPI == 1) {
+      if (t > 0) advance_copy();
+      issue_copies(t);
+    } else {
+      issue_next(t);
+    }
+  }
   unsigned slot = 0;                       // first slot of the current iteration
   const unsigned iters = k_tiles_padded / KPI;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
@@ -1040,6 +1124,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     for (unsigned it = 0; it < iters; ++it) {
+      if constexpr (KPI == 1) advance_copy();
       // After the first C tile, the K tiles of the first LEAD iterations were
       // already waited for before the previous epilogue (see below), so these
       // iterations only need the barrier; waiting on the counter here would
@@ -1057,8 +1142,12 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       // after the barrier every wave of the block would otherwise be busy with
       // their address arithmetic and the matrix cores would have nothing to do.
       auto refill_slots = [&] {
+        if constexpr (KPI == 1) {
+          issue_copies(refill);
+        } else {
 #pragma unroll
-        for (int u = 0; u < KPI; ++u) issue_next(refill + u);
+          for (int u = 0; u < KPI; ++u) issue_next(refill + u);
+        }
       };
       if constexpr (IL) {
         mma_step_interleaved<DT, BX, BY, TX, TY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
@@ -1067,7 +1156,9 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         const char *tile[KPM];
 #pragma unroll
         for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
-        if constexpr (MS == 32) {
+        if constexpr (MS == 32 && TX == 2 && TY == 2) {
+          mma_step32_ordered<DT, BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+        } else if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
         } else if constexpr (KPM == 1 && TX == 4 && TY == 4) {
           mma_step_ordered<DT, BX, BY>(tile[0], x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
