@@ -279,8 +279,6 @@ def main():
         iso_ms = e0.elapsed_time(e1) / iters
         result["isolated"] = {"gemm_ms": iso_ms, "gemm_tflops": flops / (iso_ms * 1e-3) / 1e12}
 
-    if not args.no_check:
-        result["check"] = check_result(name, a_in, b_in, c, torch)
 
     if axis_name == "interleaved":
         # The same job through ccglib's Pipeline wrapper, which here feeds the interleaved
@@ -300,6 +298,9 @@ def main():
         result["fused_pipeline"] = {
             "ms_per_step": fused_ms, "tflops": flops / (fused_ms * 1e-3) / 1e12,
             "max_abs_diff_vs_unfused": float((c2 - c).abs().max())}
+
+    if not args.no_check:
+        result["check"] = check_result(name, a_in, b_in, c, torch)
 
     if not args.no_cpu_baseline and name == "beamformer":
         import oracle as orc
