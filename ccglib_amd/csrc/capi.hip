@@ -128,11 +128,58 @@ struct ccglib_pipeline {
   hipStream_t stream;
   int type_in, type_out, c_axis;
   bool need_copyin_c;
+  // 1-bit input, one byte per sample, planar: expanded straight into the GEMM's
+  // workspace (no packed or transposed intermediates)
+  bool int1_direct = false;
   ccglib_packing_t pack_a = nullptr, pack_b = nullptr;
   ccglib_transpose_t trans_a = nullptr, trans_b = nullptr;
   ccglib_gemm_t gemm = nullptr;
   void *d_a_packed = nullptr, *d_b_packed = nullptr, *d_a_trans = nullptr, *d_b_trans = nullptr;
 };
+
+namespace {
+
+// Launch parameters of a GEMM object for the given buffers.
+void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, void *d_c,
+                      GemmParams *out) {
+  GemmParams &p = *out;
+  // C[m][n] = sum_k A[m][k] B[n][k]. The kernel wants the operand of the
+  // contiguous C axis as X: B for a row-major C, A for a column-major C (the
+  // complex product commutes, so exchanging the operands transposes C).
+  const bool row_major = (g->c_order == kRowMajor);
+  p.x = row_major ? d_b : d_a;
+  p.y = row_major ? d_a : d_b;
+  p.nx = (unsigned)(row_major ? g->N : g->M);
+  p.ny = (unsigned)(row_major ? g->M : g->N);
+  p.c = d_c;
+  p.batch = (unsigned)g->B;
+  p.k = (unsigned)g->K;
+  p.input_interleaved = g->input_interleaved;
+  if (g->input_interleaved) {
+    // a row holds K (re, im) pairs: twice the bytes, walked in 64-byte pieces
+    p.k_tiles = (unsigned)ceil_div(2 * g->K, (size_t)k_per_tile(g->type_in));
+  } else {
+    p.k_tiles = (unsigned)ceil_div(g->K, (size_t)k_per_tile(g->type_in));
+  }
+  if (p.k_tiles == 0) p.k_tiles = 1;  // K = 0: one all-zero tile keeps the epilogue uniform
+  p.x_tiles = (unsigned)ceil_div(p.nx, kTileRows);
+  p.y_tiles = (unsigned)ceil_div(p.ny, kTileRows);
+  p.type_in = g->type_in;
+  p.type_out = g->type_out;
+  p.variant = g->variant;
+  p.c_interleaved = (g->c_axis == kInterleaved);
+  p.alpha_re = g->alpha_re;
+  p.alpha_im = g->alpha_im;
+  p.beta_re = g->beta_re;
+  p.beta_im = g->beta_im;
+  // same switches as the reference's HAVE_ALPHA / HAVE_BETA (src/mma/GEMM.cpp:207-213)
+  p.have_alpha = (g->alpha_re != 1.0f || g->alpha_im != 0.0f);
+  p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
+  p.workspace = g->workspace;
+  p.workspace_bytes = g->workspace_bytes;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -240,44 +287,11 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   if (g->B == 0 || g->M == 0 || g->N == 0) return CCGLIB_OK;
   if (!d_a || !d_b || !d_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
   GemmParams p;
-  // C[m][n] = sum_k A[m][k] B[n][k]. The kernel wants the operand of the
-  // contiguous C axis as X: B for a row-major C, A for a column-major C (the
-  // complex product commutes, so exchanging the operands transposes C).
-  const bool row_major = (g->c_order == kRowMajor);
-  p.x = row_major ? d_b : d_a;
-  p.y = row_major ? d_a : d_b;
-  p.nx = (unsigned)(row_major ? g->N : g->M);
-  p.ny = (unsigned)(row_major ? g->M : g->N);
-  p.c = d_c;
-  p.batch = (unsigned)g->B;
-  p.k = (unsigned)g->K;
-  p.input_interleaved = g->input_interleaved;
-  if (g->input_interleaved) {
-    // a row holds K (re, im) pairs: twice the bytes, walked in 64-byte pieces
-    p.k_tiles = (unsigned)ceil_div(2 * g->K, (size_t)k_per_tile(g->type_in));
-    if ((uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0) {
-      return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
-                  "interleaved pipeline input must be 16-byte aligned");
-    }
-  } else {
-    p.k_tiles = (unsigned)ceil_div(g->K, (size_t)k_per_tile(g->type_in));
+  fill_gemm_params(g, d_a, d_b, d_c, &p);
+  if (g->input_interleaved && ((uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                "interleaved pipeline input must be 16-byte aligned");
   }
-  if (p.k_tiles == 0) p.k_tiles = 1;  // K = 0: one all-zero tile keeps the epilogue uniform
-  p.x_tiles = (unsigned)ceil_div(p.nx, kTileRows);
-  p.y_tiles = (unsigned)ceil_div(p.ny, kTileRows);
-  p.type_in = g->type_in;
-  p.type_out = g->type_out;
-  p.variant = g->variant;
-  p.c_interleaved = (g->c_axis == kInterleaved);
-  p.alpha_re = g->alpha_re;
-  p.alpha_im = g->alpha_im;
-  p.beta_re = g->beta_re;
-  p.beta_im = g->beta_im;
-  // same switches as the reference's HAVE_ALPHA / HAVE_BETA (src/mma/GEMM.cpp:207-213)
-  p.have_alpha = (g->alpha_re != 1.0f || g->alpha_im != 0.0f);
-  p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
-  p.workspace = g->workspace;
-  p.workspace_bytes = g->workspace_bytes;
   if (g->K == 0 && g->variant == kOpt) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "K = 0 has no tiled layout");
   }
@@ -524,6 +538,25 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   // (over the whole buffer), so what follows it sees planar data.
   const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
   do {
+    if (packing && input_complex_axis_location == kPlanar && B && M && N && K % 32 == 0) {
+      // (K in whole words, as the packed layout of the other route needs it.)
+      // The 1-bit GEMM multiplies operands expanded to 4-bit values; when its
+      // workspace holds the whole problem the expansion is done straight from
+      // the caller's bytes and the reference's pack and transpose steps
+      // (src/pipeline/Pipeline.cpp:111-121) with their buffers are not needed.
+      rc = ccglib_gemm_create(&p->gemm, B, M, N, K, device, stream, input_type, output_type,
+                              kOpt, output_complex_axis_location, c_mem_order, a_mem_order,
+                              b_mem_order, alpha_re, alpha_im, beta_re, beta_im);
+      if (rc != CCGLIB_OK) break;
+      GemmParams probe;
+      fill_gemm_params(p->gemm, nullptr, nullptr, nullptr, &probe);
+      if (gemm_int1_can_take_bytes(probe)) {
+        p->int1_direct = true;
+        break;
+      }
+      ccglib_gemm_destroy(p->gemm);
+      p->gemm = nullptr;
+    }
     if (packing) {
       const size_t num_a = B * 2 * M * K, num_b = B * 2 * N * K;  // :57-58
       if ((rc = ccglib_packing_create(&p->pack_a, num_a, kForward, device, stream,
@@ -580,6 +613,17 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
   if (!p) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pipeline handle");
   int rc;
   const void *a = d_a, *b = d_b;
+  if (p->int1_direct) {
+    ccglib_gemm *g = p->gemm;
+    if (!d_a || !d_b || !d_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+    GemmParams q;
+    fill_gemm_params(g, d_a, d_b, d_c, &q);
+    DeviceGuard guard(g->device);
+    HIP_TRY(guard.status());
+    const hipError_t e = launch_gemm_int1_from_bytes(q, g->stream);
+    if (e != hipSuccess) return fail_hip(e, "1-bit pipeline launch");
+    return CCGLIB_OK;
+  }
   if (p->pack_a) {  // src/pipeline/Pipeline.cpp:111-114
     if ((rc = ccglib_packing_run(p->pack_a, a, p->d_a_packed))) return rc;
     if ((rc = ccglib_packing_run(p->pack_b, b, p->d_b_packed))) return rc;

@@ -85,6 +85,12 @@ struct GemmParams {
 // Bytes of workspace with which the 1-bit GEMM of this size runs in one pass.
 size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k);
 
+// 1-bit GEMM whose operands p.x / p.y are one byte per sample, planar
+// [batch][2][rows][k] (the pipeline's input): expanded straight into the
+// workspace and multiplied on the fp4 MFMA. Only when gemm_int1_can_take_bytes.
+bool gemm_int1_can_take_bytes(const GemmParams &p);
+hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream);
+
 hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream);
 hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream);
 

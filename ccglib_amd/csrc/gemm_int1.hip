@@ -198,9 +198,10 @@ __device__ __forceinline__ unsigned spread8(unsigned x) {
   return x;
 }
 
-// One thread per 32 samples of one row: one word of bits in, 16 bytes out. A
-// wave reads 4 source rows (256 bytes contiguous) and writes 4 rows x 64 bytes
-// (256 bytes contiguous) into each of four K tiles of the expanded layout.
+// A thread takes word c (of four) of each of the four 128-sample K tiles that a
+// 64-byte row of the 1-bit layout spans: four 4-byte loads in flight per thread
+// (with one, the kernel is bound by the latency of its reads), and every store
+// instruction of a wave writes 16 rows x 64 bytes = 1 KiB contiguous.
 // TILED: the source is the 1-bit tiled layout (tiles of 512 samples); otherwise
 // planar rows of k_words words.
 template <bool TILED>
@@ -208,41 +209,111 @@ __global__ __launch_bounds__(256) void expand_int1_to_fp4(const char *__restrict
                                                           char *__restrict__ dst, unsigned rows, unsigned row_tiles,
                                                           unsigned k, unsigned k1_tiles,
                                                           unsigned k4_tiles, unsigned k_words) {
-  // blockIdx.x: (batch, row tile, source K tile), uniform per block; blockIdx.y
-  // and the thread index: (plane, row, chunk, word) of that tile
-  const unsigned t = blockIdx.y * 256 + threadIdx.x;
-  const unsigned j = t & 3, c = (t >> 2) & 3, row = (t >> 4) & 127, plane = (t >> 11) & 1;
+  // blockIdx.x: (batch, row tile, source K tile of 512 samples); blockIdx.y: (plane, half of the 128 rows)
+  const unsigned c = threadIdx.x & 3, row = (blockIdx.y & 1) * 64 + (threadIdx.x >> 2);
+  const unsigned plane = blockIdx.y >> 1;
   const unsigned kt1 = blockIdx.x % k1_tiles;
   const unsigned rest = blockIdx.x / k1_tiles;
   const unsigned rt = rest % row_tiles;
   const size_t b = rest / row_tiles;
-  const unsigned k4 = 4 * kt1 + c;          // K tile of the expanded layout (128 samples)
-  if (k4 >= k4_tiles) return;
-  unsigned bits = 0;
+  unsigned w[4] = {0, 0, 0, 0};
   if constexpr (TILED) {
-    bits = *reinterpret_cast<const unsigned *>(src + ((b * row_tiles + rt) * k1_tiles + kt1) * kTileBytes +
-                                               plane * kTilePlaneBytes + row * kTileRowBytes + c * 16 +
-                                               j * 4);
+    const unsigned *p = reinterpret_cast<const unsigned *>(
+                            src + ((b * row_tiles + rt) * k1_tiles + kt1) * kTileBytes +
+                            plane * kTilePlaneBytes + row * kTileRowBytes) + c;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) w[s] = p[4 * s];
   } else {
     const unsigned r = rt * kTileRows + row;
-    if (r < rows && 4 * k4 + j < k_words) {
-      bits = reinterpret_cast<const unsigned *>(src)[((b * 2 + plane) * rows + r) * (size_t)k_words +
-                                                     4 * k4 + j];
+    if (r < rows) {
+      const unsigned *p = reinterpret_cast<const unsigned *>(src) +
+                          ((b * 2 + plane) * rows + r) * (size_t)k_words + 16 * kt1 + c;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (16 * kt1 + 4 * s + c < k_words) w[s] = p[4 * s];
+      }
     }
   }
-  // samples of this word that exist: the others become 0.0
-  const unsigned first = k4 * 128 + 32 * j;
-  const unsigned n = first >= k ? 0u : (k - first >= 32 ? 32u : k - first);
-  const unsigned valid = n == 32 ? 0xffffffffu : ((1u << n) - 1u);
-  const unsigned w = bits & valid;
-  uint4_t o;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    o[q] = (spread8((w >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
+  for (int s = 0; s < 4; ++s) {
+    const unsigned k4 = 4 * kt1 + s;          // K tile of the expanded layout (128 samples)
+    if (k4 >= k4_tiles) break;
+    // samples of this word that exist: the others become 0.0
+    const unsigned first = k4 * 128 + 32 * c;
+    const unsigned n = first >= k ? 0u : (k - first >= 32 ? 32u : k - first);
+    const unsigned valid = n == 32 ? 0xffffffffu : ((1u << n) - 1u);
+    const unsigned ws = w[s] & valid;
+    uint4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o[q] = (spread8((ws >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
+    }
+    __builtin_nontemporal_store(
+        o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
+                                       plane * kTilePlaneBytes + row * kTileRowBytes + 16 * c));
   }
-  __builtin_nontemporal_store(
-      o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
-                                     plane * kTilePlaneBytes + row * kTileRowBytes + 16 * j));
+}
+
+// The same expansion straight from one byte per sample (the pipeline's input:
+// any non-zero byte is a 1, kernels/packing_kernel.cu:14-22), which saves the
+// packed and the transposed intermediate of the pack -> transpose -> expand
+// sequence. Planar input [batch][2][rows][k]; a thread takes 32 samples of each
+// of four K tiles (eight 16-byte loads in flight) and writes four 16-byte pieces;
+// every store instruction of a wave writes 1 KiB contiguous.
+__device__ __forceinline__ unsigned nonzero_bits_of4(unsigned x) {   // 4 bytes -> 4 bits
+  const unsigned nz = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
+  return (((nz >> 7) * 0x00204081u) >> 21) & 0xfu;
+}
+__device__ __forceinline__ unsigned nonzero_bits_of16(uint4_t v) {
+  return nonzero_bits_of4(v[0]) | (nonzero_bits_of4(v[1]) << 4) | (nonzero_bits_of4(v[2]) << 8) |
+         (nonzero_bits_of4(v[3]) << 12);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *__restrict__ src,
+                                                           char *__restrict__ dst, unsigned rows,
+                                                           unsigned row_tiles, unsigned k,
+                                                           unsigned k4_tiles) {
+  // blockIdx: x = group of four K tiles of 128 samples, y = block of 64 rows, z = (batch, plane);
+  // a thread takes quarter c of each of the four K tiles (eight 16-byte loads in flight)
+  const unsigned c = threadIdx.x & 3, row_in_tile = (blockIdx.y & 1) * 64 + (threadIdx.x >> 2);
+  const unsigned rt = blockIdx.y >> 1;
+  const size_t b = blockIdx.z >> 1;
+  const unsigned plane = blockIdx.z & 1;
+  const unsigned r = rt * kTileRows + row_in_tile;
+  const unsigned char *row_ptr = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
+  unsigned bits[4], n[4];
+  uint4_t v[4][2];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const unsigned k0 = (4 * blockIdx.x + s) * 128 + c * 32;
+    n[s] = (r < rows && k0 < k) ? (k - k0 < 32 ? k - k0 : 32) : 0;
+    if (VEC && n[s] == 32) {
+      v[s][0] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr + k0));
+      v[s][1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr + k0) + 1);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const unsigned k4 = 4 * blockIdx.x + s;
+    if (k4 >= k4_tiles) break;
+    const unsigned k0 = k4 * 128 + c * 32;
+    if (VEC && n[s] == 32) {
+      bits[s] = nonzero_bits_of16(v[s][0]) | (nonzero_bits_of16(v[s][1]) << 16);
+    } else {
+      bits[s] = 0;
+      for (unsigned i = 0; i < n[s]; ++i) bits[s] |= (row_ptr[k0 + i] != 0 ? 1u : 0u) << i;
+    }
+    const unsigned valid = n[s] == 32 ? 0xffffffffu : ((1u << n[s]) - 1u);
+    uint4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o[q] = (spread8((bits[s] >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
+    }
+    __builtin_nontemporal_store(
+        o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
+                                       plane * kTilePlaneBytes + row_in_tile * kTileRowBytes + 16 * c));
+  }
 }
 
 // Largest K for which every partial sum (at most 2 K in magnitude) is exact in fp32.
@@ -273,7 +344,7 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
       char *dst = which ? ws_y : ws_x;
       const size_t blocks = nb * row_tiles * k1_tiles;
       if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-      const dim3 grid((unsigned)blocks, 16);
+      const dim3 grid((unsigned)blocks, 4);
       if (tiled) {
         hipLaunchKernelGGL(expand_int1_to_fp4<true>, grid, dim3(256), 0, stream, src, dst, rows,
                            row_tiles, p.k, k1_tiles, k4_tiles, k_words);
@@ -298,6 +369,43 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
 }
 
 }  // namespace
+
+bool gemm_int1_can_take_bytes(const GemmParams &p) {
+  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return false;
+  if (p.workspace_bytes < gemm_int1_workspace_bytes(p.batch, p.nx, p.ny, p.k)) return false;
+  return p.batch <= 32767 && 2 * (size_t)p.x_tiles <= 65535 && 2 * (size_t)p.y_tiles <= 65535;
+}
+
+hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
+  if (!gemm_int1_can_take_bytes(p)) return hipErrorInvalidValue;
+  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
+  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
+  char *ws_x = static_cast<char *>(p.workspace);
+  char *ws_y = ws_x + p.batch * x_bytes;
+  for (int which = 0; which < 2; ++which) {
+    const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+    const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
+    char *dst = which ? ws_y : ws_x;
+    const dim3 grid((unsigned)ceil_div(k4_tiles, 4), 2 * row_tiles, 2 * p.batch);
+    const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
+    if (vec) {
+      hipLaunchKernelGGL(expand_bytes_to_fp4<true>, grid, dim3(256), 0, stream, src, dst, rows,
+                         row_tiles, p.k, k4_tiles);
+    } else {
+      hipLaunchKernelGGL(expand_bytes_to_fp4<false>, grid, dim3(256), 0, stream, src, dst, rows,
+                         row_tiles, p.k, k4_tiles);
+    }
+  }
+  GemmParams q = p;
+  q.x = ws_x;
+  q.y = ws_y;
+  q.k_tiles = k4_tiles;
+  q.type_in = kFp4Sign;
+  q.variant = kOpt;
+  q.input_interleaved = 0;
+  if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
+  return hipGetLastError();
+}
 
 size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k) {
   if (k == 0 || k > kMaxMfmaK) return 0;

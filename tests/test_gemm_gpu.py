@@ -1,6 +1,9 @@
 """GPU parity tests of the complex GEMM against the CPU oracle, through the C ABI
 (ccglib_amd.GEMM / Transpose are thin ctypes bindings). Shapes and cases follow
 the reference's test/gemm/mma.cpp."""
+import json
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -85,27 +88,30 @@ def float_case(B, M, N, K, tin, tout, variant, c_axis, c_order, signed=True, alp
 
 # ---- reference known answers, through the GPU --------------------------------------
 
-KAT_A = [1, 2, 3, 4, 5, 6, 6, 5, 4, 3, 2, 1]
-KAT_B = [1, 2, 3, 4, 4, 3, 2, 1]
+# tests/golden/reference_kats.json: the vectors of the reference's test/gemm/reference.cpp
+KATS = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                   "reference_kats.json")))
+KAT_A, KAT_B = KATS["float"]["a"], KATS["float"]["b"]
 
 
 @pytest.mark.parametrize("tin", [VT.float16, VT.bfloat16, VT.float32])
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
 def test_kat_float(tin, variant):
-    qa, qb = quantize(np.array(KAT_A), tin), quantize(np.array(KAT_B), tin)
-    c = run_gemm(qa, qb, 1, 3, 2, 2, tin, VT.float32, variant)
-    assert c.reshape(-1).tolist() == [-34, -6, -14, 14, 6, 34, 26, 42, 34, 34, 42, 26]
-    c = run_gemm(qa, qb, 1, 3, 2, 2, tin, VT.float32, variant, c_order=COL)
-    assert c.reshape(-1).tolist() == [-34, -14, 6, -6, 14, 34, 26, 34, 42, 42, 34, 26]
+    k = KATS["float"]
+    qa, qb = quantize(np.array(k["a"]), tin), quantize(np.array(k["b"]), tin)
+    c = run_gemm(qa, qb, 1, k["M"], k["N"], k["K"], tin, VT.float32, variant)
+    assert c.reshape(-1).tolist() == k["c_row_major"]
+    c = run_gemm(qa, qb, 1, k["M"], k["N"], k["K"], tin, VT.float32, variant, c_order=COL)
+    assert c.reshape(-1).tolist() == k["c_col_major"]
 
 
 def test_kat_alpha_beta_fp16():
-    seq = list(range(16)) + list(range(16, 0, -1))
-    q = quantize(np.array(seq), VT.float16)
-    c_in = np.array([0, 1, 2, 3, 4, 3, 2, 1], dtype=np.float32)
-    c = run_gemm(q, q.copy(), 1, 2, 2, 8, VT.float16, VT.float32, cc.Variant.basic,
-                 alpha=0.5 + 2.5j, beta=0.25 - 1.5j, c_in=c_in)
-    assert c.reshape(-1).tolist() == [-2110, -3039.25, -3040.5, -1409.75, -2571, 275.25, 273.5, 2607.75]
+    k = KATS["alpha_beta_float16"]
+    c = run_gemm(quantize(np.array(k["a"]), VT.float16), quantize(np.array(k["b"]), VT.float16), 1,
+                 k["M"], k["N"], k["K"], VT.float16, VT.float32, cc.Variant.basic,
+                 alpha=complex(*k["alpha"]), beta=complex(*k["beta"]),
+                 c_in=np.array(k["c_in"], dtype=np.float32))
+    assert c.reshape(-1).tolist() == k["c_row_major"]
 
 
 def test_all_ones_closed_form():
@@ -265,17 +271,23 @@ def int1_case(B, M, N, K, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0, 
     assert np.array_equal(got.reshape(want.shape), want)
 
 
-def test_kat_int1():
-    a = np.array([4007499276, 2587246816, 2368114480, 2180517764], dtype=np.uint32)
-    b = np.array([3172811225, 4156143586, 144478092, 808068269], dtype=np.uint32)
-    for c_in, alpha, beta, want in [
-            (np.zeros(8, np.int32), 1, 0, [-8, 8, -10, -6, 8, -12, -6, 6]),
-            (np.arange(1, 9, dtype=np.int32), 2 + 3j, -1 + 2j, [-51, 38, -19, -50, -11, -2, -43, -6])]:
-        d_a, d_b, d_c = to_device(a), to_device(b), to_device(c_in)
-        cc.GEMM(1, 2, 2, 32, 0, stream(), cc.Precision(VT.int1, VT.int32), cc.Variant.basic, PLANAR,
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_kat_int1(variant, int1_kernel):
+    for k, c_in, alpha, beta in [
+            (KATS["int1"], np.zeros(8, np.int32), 1, 0),
+            (KATS["alpha_beta_int1"], np.array(KATS["alpha_beta_int1"]["c_in"], dtype=np.int32),
+             complex(*KATS["alpha_beta_int1"]["alpha"]), complex(*KATS["alpha_beta_int1"]["beta"]))]:
+        a, b = np.array(k["a"], dtype=np.uint32), np.array(k["b"], dtype=np.uint32)
+        if variant == cc.Variant.opt:
+            d_a = transpose_operand(a, 1, k["M"], k["K"], VT.int1)
+            d_b = transpose_operand(b, 1, k["N"], k["K"], VT.int1)
+        else:
+            d_a, d_b = to_device(a), to_device(b)
+        d_c = to_device(c_in)
+        cc.GEMM(1, k["M"], k["N"], k["K"], 0, stream(), cc.Precision(VT.int1, VT.int32), variant, PLANAR,
                 ROW, ROW, COL, alpha, beta).Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
         torch.cuda.synchronize()
-        assert to_host(d_c, np.int32).tolist() == want
+        assert to_host(d_c, np.int32).tolist() == k["c_row_major"]
 
 
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])

@@ -19,55 +19,58 @@ def enc(vals, vtype):
     return v
 
 
-# ---- reference known-answer tests (test/gemm/reference.cpp) -----------------
+# ---- reference known-answer tests (tests/golden/reference_kats.json) --------
 
-KAT_A = [1, 2, 3, 4, 5, 6, 6, 5, 4, 3, 2, 1]          # :27-33, a(2,3,2)
-KAT_B = [1, 2, 3, 4, 4, 3, 2, 1]                      # :35-39, b(2,2,2)
-KAT_C_ROW = [-34, -6, -14, 14, 6, 34, 26, 42, 34, 34, 42, 26]   # :41-42
-KAT_C_COL = [-34, -14, 6, -6, 14, 34, 26, 34, 42, 42, 34, 26]   # :44-45
+import json
+import os
+
+KATS = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                   "reference_kats.json")))
 
 
 @pytest.mark.parametrize("vtype", [orc.FLOAT16, orc.BFLOAT16, orc.FLOAT32])
 def test_kat_float(vtype):
-    a, b = enc(KAT_A, vtype), enc(KAT_B, vtype)
-    c = orc.gemm(a, b, 3, 2, 2, vtype, orc.FLOAT32, orc.ROW_MAJOR)
-    assert c.reshape(-1).tolist() == KAT_C_ROW
-    c = orc.gemm(a, b, 3, 2, 2, vtype, orc.FLOAT32, orc.COL_MAJOR)
-    assert c.reshape(-1).tolist() == KAT_C_COL
+    k = KATS["float"]
+    a, b = enc(k["a"], vtype), enc(k["b"], vtype)
+    c = orc.gemm(a, b, k["M"], k["N"], k["K"], vtype, orc.FLOAT32, orc.ROW_MAJOR)
+    assert c.reshape(-1).tolist() == k["c_row_major"]
+    c = orc.gemm(a, b, k["M"], k["N"], k["K"], vtype, orc.FLOAT32, orc.COL_MAJOR)
+    assert c.reshape(-1).tolist() == k["c_col_major"]
 
 
-INT1_A = np.array([4007499276, 2587246816, 2368114480, 2180517764], dtype=np.uint32)  # :73-74
-INT1_B = np.array([3172811225, 4156143586, 144478092, 808068269], dtype=np.uint32)    # :75-76
+INT1_A = np.array(KATS["int1"]["a"], dtype=np.uint32)
+INT1_B = np.array(KATS["int1"]["b"], dtype=np.uint32)
 
 
 def test_kat_int1():
-    c = orc.gemm(INT1_A, INT1_B, 2, 2, 32, orc.INT1, orc.INT32, orc.ROW_MAJOR,
+    k = KATS["int1"]
+    c = orc.gemm(INT1_A, INT1_B, k["M"], k["N"], k["K"], orc.INT1, orc.INT32, orc.ROW_MAJOR,
                  c_in=np.zeros(8, np.int32))
-    assert c.reshape(-1).tolist() == [-8, 8, -10, -6, 8, -12, -6, 6]      # :77-78
-    c = orc.gemm(INT1_A, INT1_B, 2, 2, 32, orc.INT1, orc.INT32, orc.COL_MAJOR,
+    assert c.reshape(-1).tolist() == k["c_row_major"]
+    c = orc.gemm(INT1_A, INT1_B, k["M"], k["N"], k["K"], orc.INT1, orc.INT32, orc.COL_MAJOR,
                  c_in=np.zeros(8, np.int32))
-    assert c.reshape(-1).tolist() == [-8, -10, 8, -6, 8, -6, -12, 6]      # :79-80
+    assert c.reshape(-1).tolist() == k["c_col_major"]
 
 
 def test_kat_alpha_beta_fp16():
-    seq = list(range(16)) + list(range(16, 0, -1))                         # :102-107
-    a = enc(seq, orc.FLOAT16)
-    c_in = np.array([0, 1, 2, 3, 4, 3, 2, 1], dtype=np.float32)             # :108
-    c = orc.gemm(a, a.copy(), 2, 2, 8, orc.FLOAT16, orc.FLOAT32, orc.ROW_MAJOR,
-                 alpha=0.5 + 2.5j, beta=0.25 - 1.5j, c_in=c_in)
-    assert c.reshape(-1).tolist() == [-2110, -3039.25, -3040.5, -1409.75,
-                                      -2571, 275.25, 273.5, 2607.75]        # :109-110
+    k = KATS["alpha_beta_float16"]
+    c = orc.gemm(enc(k["a"], orc.FLOAT16), enc(k["b"], orc.FLOAT16), k["M"], k["N"], k["K"],
+                 orc.FLOAT16, orc.FLOAT32, orc.ROW_MAJOR, alpha=complex(*k["alpha"]),
+                 beta=complex(*k["beta"]), c_in=np.array(k["c_in"], dtype=np.float32))
+    assert c.reshape(-1).tolist() == k["c_row_major"]
 
 
 def test_kat_alpha_beta_int1():
-    c_in = np.arange(1, 9, dtype=np.int32)                                  # :132
-    c = orc.gemm(INT1_A, INT1_B, 2, 2, 32, orc.INT1, orc.INT32, orc.ROW_MAJOR,
-                 alpha=2 + 3j, beta=-1 + 2j, c_in=c_in)
-    assert c.reshape(-1).tolist() == [-51, 38, -19, -50, -11, -2, -43, -6]  # :133-134
+    k = KATS["alpha_beta_int1"]
+    c = orc.gemm(np.array(k["a"], dtype=np.uint32), np.array(k["b"], dtype=np.uint32), k["M"],
+                 k["N"], k["K"], orc.INT1, orc.INT32, orc.ROW_MAJOR, alpha=complex(*k["alpha"]),
+                 beta=complex(*k["beta"]), c_in=np.array(k["c_in"], dtype=np.int32))
+    assert c.reshape(-1).tolist() == k["c_row_major"]
 
 
 def test_ceildiv():
-    assert orc.ceildiv(10, 5) == 2 and orc.ceildiv(16, 5) == 4              # test/helper.cpp:7-9
+    for a, b, want in KATS["ceildiv"]["cases"]:
+        assert orc.ceildiv(a, b) == want
 
 
 # ---- closed forms and independent routines -----------------------------------

@@ -100,6 +100,48 @@ def test_pipeline_int1(variant):
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
+@pytest.mark.parametrize("mode", ["direct", "popcount", "capped_workspace"])
+@pytest.mark.parametrize("M,N,K,c_order", [(130, 70, 992, ROW), (64, 200, 96, COL), (20, 30, 32, ROW),
+                                           (256, 128, 2048, COL)])
+def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
+    # Planar one-byte-per-sample input is expanded straight into the 1-bit GEMM's
+    # workspace ("direct"); without a (whole) workspace the pipeline packs and
+    # transposes as the reference does. Any non-zero byte is a 1 bit.
+    monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
+    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
+    if mode == "popcount":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
+    elif mode == "capped_workspace":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+    B = 3
+    rng = np.random.default_rng(M + K)
+    a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8)
+    # other non-zero values count as 1 too
+    a_in = a_bits * rng.integers(1, 256, a_bits.size, dtype=np.uint8)
+    b_in = b_bits * rng.integers(1, 256, b_bits.size, dtype=np.uint8)
+    alpha, beta = -1 + 2j, 3 + 1j
+    c_in = rng.integers(-1000, 1000, B * 2 * M * N).astype(np.int32)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, c_order, VT.int1, VT.int32,
+                    cc.Variant.opt, alpha, beta)
+    d_a, d_b, d_c = to_device(a_in), to_device(b_in), to_device(c_in)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())     # beta != 0: applied twice
+    torch.cuda.synchronize()
+    pa, pb = pack_rows(a_bits, B, M, K), pack_rows(b_bits, B, N, K)
+    once = orc.gemm(pa, pb, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, c_in)
+    want = orc.gemm(pa, pb, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, once.reshape(-1))
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+
+
+def pack_rows(bits, B, rows, K):
+    """One byte per sample [B][2][rows][K] -> rows of whole 32-bit words, LSB first."""
+    kw = (K + 31) // 32
+    padded = np.zeros((B * 2 * rows, kw * 32), dtype=np.uint8)
+    padded[:, :K] = bits.reshape(B * 2 * rows, K)
+    return np.packbits(padded, axis=1, bitorder="little").view(np.uint32).reshape(-1)
+
+
 def interleaved(q, B, rows, K):
     return np.ascontiguousarray(q.reshape(B, 2, rows, K).transpose(0, 2, 3, 1)).reshape(-1)
 
