@@ -137,6 +137,9 @@ def main():
                     help="also launch a plain 1 GiB device copy (for scaling rocprofv3 HBM counters)")
     ap.add_argument("--isolated", action="store_true",
                     help="also time the GEMM launched back to back outside the step")
+    ap.add_argument("--host", action="store_true",
+                    help="also time Pipeline's host-pointer Run on page-locked buffers (copies over "
+                         "PCIe in both directions included; never part of `value`)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the batch axis "
@@ -317,6 +320,37 @@ def main():
             "ms_per_step": fused_ms, "tops": flops / (fused_ms * 1e-3) / 1e12,
             "identical_to_unfused": bool(torch.equal(c2, c))}
         del pipe, c2
+
+    if args.host:
+        # Host buffers in, host buffer out: the pipeline's host-pointer Run, which moves
+        # chunks of batches over a few streams so that copies in, kernels and copies out overlap.
+        in_axis = AX.complex_interleaved if axis_name == "interleaved" else AX.complex_planar
+        pipe = cc.Pipeline(B, M, N, K, 0, stream, in_axis, AX.complex_planar, MO.row_major,
+                           MO.col_major, MO.row_major, tin, tout, cc.Variant.opt)
+        h_a = torch.empty(a_in.numel() * a_in.element_size(), dtype=torch.uint8, pin_memory=True)
+        h_b = torch.empty(b_in.numel() * b_in.element_size(), dtype=torch.uint8, pin_memory=True)
+        h_c = torch.empty(c.numel() * c.element_size(), dtype=torch.uint8, pin_memory=True)
+        h_a.copy_(a_in.view(torch.uint8).reshape(-1))
+        h_b.copy_(b_in.view(torch.uint8).reshape(-1))
+        torch.cuda.synchronize()
+        reps = 3
+        pipe.RunHost(h_a.data_ptr(), h_b.data_ptr(), h_c.data_ptr())
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            pipe.RunHost(h_a.data_ptr(), h_b.data_ptr(), h_c.data_ptr())
+        host_ms = (time.perf_counter() - t0) * 1e3 / reps
+        moved = h_a.numel() + h_b.numel() + h_c.numel()
+        c_dev = torch.empty_like(c)
+        pipe.Run(a_in.data_ptr(), b_in.data_ptr(), c_dev.data_ptr())
+        torch.cuda.synchronize()
+        same = bool(torch.equal(h_c, c_dev.view(torch.uint8).reshape(-1).cpu()))
+        del c_dev
+        result["host_pipeline"] = {
+            "ms_per_run": host_ms, "tflops": flops / (host_ms * 1e-3) / 1e12,
+            "host_bytes_in": h_a.numel() + h_b.numel(), "host_bytes_out": h_c.numel(),
+            "pcie_gbs_both_directions": moved / host_ms / 1e6,
+            "identical_to_device_run": same}
+        del pipe, h_a, h_b, h_c
 
     if not args.no_check:
         result["check"] = check_result(name, a_in, b_in, c, torch)

@@ -3,6 +3,7 @@
 // behaviour mirrors the reference classes it replaces: src/mma/GEMM.cpp,
 // src/transpose/Transpose.cpp, src/packing/Packing.cpp,
 // src/pipeline/Pipeline.cpp.
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -135,6 +136,22 @@ struct ccglib_pipeline {
   ccglib_transpose_t trans_a = nullptr, trans_b = nullptr;
   ccglib_gemm_t gemm = nullptr;
   void *d_a_packed = nullptr, *d_b_packed = nullptr, *d_a_trans = nullptr, *d_b_trans = nullptr;
+  // What the object was created with, for the batch-chunked host path below.
+  int in_axis = 0, a_order = 0, b_order = 0, c_order = 0, variant = 0;
+  float alpha_re = 1, alpha_im = 0, beta_re = 0, beta_im = 0;
+  // Host-pointer Run in chunks of whole batches on a few lanes, each a stream with
+  // a pipeline of chunk_B batches and device buffers for one chunk, so that the
+  // copies to the device, the kernels and the copies back of different chunks
+  // overlap. Created by the first host Run that is large enough to use them.
+  // (two: with three or four the copies of the 1.75 GB beamformer job took 25-35
+  // ms instead of 23)
+  static constexpr int kHostLanes = 2;
+  size_t chunk_B = 0;
+  ccglib_pipeline *lane[kHostLanes] = {};
+  ccglib_pipeline *lane_tail = nullptr;   // for a last chunk of fewer batches
+  hipStream_t lane_stream[kHostLanes] = {};
+  void *lane_a[kHostLanes] = {}, *lane_b[kHostLanes] = {}, *lane_c[kHostLanes] = {};
+  hipEvent_t caller_ready = nullptr;
 };
 
 namespace {
@@ -480,6 +497,38 @@ int ccglib_packing_destroy(ccglib_packing_t k) {
 
 /* ------------------------------ Pipeline -------------------------------- */
 
+}  // extern "C"
+
+namespace {
+
+// Frees what the chunked host path of a pipeline holds.
+void destroy_host_lanes(ccglib_pipeline *p) {
+  if (!p->caller_ready && !p->lane_stream[0]) return;
+  DeviceGuard guard(p->device);
+  for (int l = 0; l < ccglib_pipeline::kHostLanes; ++l) {
+    if (p->lane_stream[l]) (void)hipStreamSynchronize(p->lane_stream[l]);
+  }
+  ccglib_pipeline_destroy(p->lane_tail);
+  p->lane_tail = nullptr;
+  for (int l = 0; l < ccglib_pipeline::kHostLanes; ++l) {
+    ccglib_pipeline_destroy(p->lane[l]);
+    if (p->lane_a[l]) (void)hipFree(p->lane_a[l]);
+    if (p->lane_b[l]) (void)hipFree(p->lane_b[l]);
+    if (p->lane_c[l]) (void)hipFree(p->lane_c[l]);
+    if (p->lane_stream[l]) (void)hipStreamDestroy(p->lane_stream[l]);
+    p->lane[l] = nullptr;
+    p->lane_a[l] = p->lane_b[l] = p->lane_c[l] = nullptr;
+    p->lane_stream[l] = nullptr;
+  }
+  if (p->caller_ready) (void)hipEventDestroy(p->caller_ready);
+  p->caller_ready = nullptr;
+  p->chunk_B = 0;
+}
+
+}  // namespace
+
+extern "C" {
+
 int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
   if (!p) return CCGLIB_OK;
   {
@@ -489,6 +538,7 @@ int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
     if (p->d_a_trans) (void)hipFree(p->d_a_trans);
     if (p->d_b_trans) (void)hipFree(p->d_b_trans);
   }
+  destroy_host_lanes(p);
   ccglib_packing_destroy(p->pack_a);
   ccglib_packing_destroy(p->pack_b);
   ccglib_transpose_destroy(p->trans_a);
@@ -525,6 +575,15 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   p->type_out = output_type;
   p->c_axis = output_complex_axis_location;
   p->need_copyin_c = (beta_re != 0.0f || beta_im != 0.0f);  // src/pipeline/Pipeline.cpp:138
+  p->in_axis = input_complex_axis_location;
+  p->a_order = a_mem_order;
+  p->b_order = b_mem_order;
+  p->c_order = c_mem_order;
+  p->variant = variant;
+  p->alpha_re = alpha_re;
+  p->alpha_im = alpha_im;
+  p->beta_re = beta_re;
+  p->beta_im = beta_im;
   int rc = CCGLIB_OK;
   const bool packing = (input_type == kInt1);   // src/pipeline/Pipeline.cpp:52
   // Interleaved 8/16-bit input whose rows are whole 16-byte chunks is fed to the
@@ -639,6 +698,74 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
   return ccglib_gemm_run(p->gemm, a, b, d_c);  // :123-125
 }
 
+}  // extern "C"
+
+namespace {
+
+// Batches per chunk of the overlapped host path, or 0 when the problem is run
+// in one piece: a single batch, less than 8 MiB to move, or 1-bit interleaved
+// input (its packing moves the real samples of the *whole* buffer in front,
+// src/pipeline/Pipeline.cpp:111-114 with kernels/packing_kernel.cu:15-22, so a
+// batch is not a contiguous piece of work there). Chunks of about 32 MiB keep
+// copies in both directions in flight at once (sizes from 8 to 64 MiB measured
+// the same, 128 MiB 7 % slower);
+// CCGLIB_AMD_HOST_CHUNK_BYTES overrides that size.
+size_t host_chunk_batches(const ccglib_pipeline *p, size_t bytes_total) {
+  if (p->B < 2 || (p->type_in == kInt1 && p->in_axis == kInterleaved)) return 0;
+  size_t target = (size_t)32 << 20;
+  const char *env = std::getenv("CCGLIB_AMD_HOST_CHUNK_BYTES");
+  if (env && *env) {
+    target = std::max<size_t>(1, std::strtoull(env, nullptr, 10));
+  } else if (bytes_total < ((size_t)8 << 20)) {
+    return 0;
+  }
+  const size_t per_batch = std::max<size_t>(1, bytes_total / p->B);
+  const size_t chunk = std::max<size_t>(1, target / per_batch);
+  return chunk < p->B ? chunk : ceil_div(p->B, 2);   // the last chunk may hold fewer batches
+}
+
+// Creates the lanes of the chunked host path; an object whose chunk size
+// changed (the environment variable) gets new ones.
+int make_host_lanes(ccglib_pipeline *p, size_t chunk, size_t bytes_a, size_t bytes_b,
+                    size_t bytes_c) {
+  constexpr int kLanes = ccglib_pipeline::kHostLanes;
+  if (p->chunk_B == chunk) return CCGLIB_OK;
+  destroy_host_lanes(p);
+  const size_t chunks = ceil_div(p->B, chunk), tail = p->B - (chunks - 1) * chunk;
+  hipError_t e = hipEventCreateWithFlags(&p->caller_ready, hipEventDisableTiming);
+  for (int l = 0; l < kLanes && e == hipSuccess; ++l) {
+    e = hipStreamCreateWithFlags(&p->lane_stream[l], hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipMalloc(&p->lane_a[l], bytes_a / p->B * chunk + 16);
+    if (e == hipSuccess) e = hipMalloc(&p->lane_b[l], bytes_b / p->B * chunk + 16);
+    if (e == hipSuccess) e = hipMalloc(&p->lane_c[l], bytes_c / p->B * chunk + 16);
+  }
+  if (e != hipSuccess) {
+    destroy_host_lanes(p);
+    return fail_hip(e, "pipeline host lanes");
+  }
+  for (int l = 0; l <= kLanes; ++l) {
+    if (l == kLanes && tail == chunk) break;
+    // the last chunk is number chunks - 1 and runs on that lane's stream
+    const int rc = ccglib_pipeline_create(
+        l < kLanes ? &p->lane[l] : &p->lane_tail, l < kLanes ? chunk : tail, p->M, p->N, p->K,
+        p->device, p->lane_stream[l < kLanes ? l : (int)((chunks - 1) % kLanes)], p->in_axis,
+        p->c_axis, p->a_order, p->b_order, p->c_order, p->type_in, p->type_out, p->variant,
+        p->alpha_re, p->alpha_im, p->beta_re, p->beta_im);
+    if (rc != CCGLIB_OK) {
+      const std::string keep = g_last_error;
+      destroy_host_lanes(p);
+      g_last_error = keep;
+      return rc;
+    }
+  }
+  p->chunk_B = chunk;
+  return CCGLIB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
 int ccglib_pipeline_run_host(ccglib_pipeline_t p, const void *h_a, const void *h_b, void *h_c) {
   if (!p) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pipeline handle");
   if (!h_a || !h_b || !h_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null host pointer");
@@ -650,9 +777,54 @@ int ccglib_pipeline_run_host(ccglib_pipeline_t p, const void *h_a, const void *h
   if (bytes_c == 0) return CCGLIB_OK;
   DeviceGuard guard(p->device);
   HIP_TRY(guard.status());
-  void *d_a = nullptr, *d_b = nullptr, *d_c = nullptr;
   int rc = CCGLIB_OK;
-  hipError_t e = hipMalloc(&d_a, bytes_a ? bytes_a : 16);
+  hipError_t e = hipSuccess;
+
+  const size_t chunk = host_chunk_batches(p, bytes_a + bytes_b + bytes_c);
+  if (chunk) {
+    // Chunks of whole batches go round the lanes; within a lane the
+    // stream keeps copy in -> kernels -> copy out of one chunk, and the next use
+    // of the lane's buffers, in order. With pinned host memory every call below
+    // returns at once and the lanes run against each other (the copies of one
+    // with the kernels and the opposite copies of the other); with pageable
+    // memory the copies block the host, and the result is the same.
+    if ((rc = make_host_lanes(p, chunk, bytes_a, bytes_b, bytes_c))) return rc;
+    const size_t chunks = ceil_div(p->B, chunk);
+    const size_t batch_a = bytes_a / p->B, batch_b = bytes_b / p->B, batch_c = bytes_c / p->B;
+    // work the caller queued on its stream comes first
+    e = hipEventRecord(p->caller_ready, p->stream);
+    for (int l = 0; l < ccglib_pipeline::kHostLanes && e == hipSuccess; ++l) {
+      e = hipStreamWaitEvent(p->lane_stream[l], p->caller_ready, 0);
+    }
+    for (size_t i = 0; i < chunks && e == hipSuccess && rc == CCGLIB_OK; ++i) {
+      const int l = (int)(i % ccglib_pipeline::kHostLanes);
+      hipStream_t s = p->lane_stream[l];
+      const size_t batches = std::min(chunk, p->B - i * chunk);
+      ccglib_pipeline *lane = batches == chunk ? p->lane[l] : p->lane_tail;
+      const size_t ca = batches * batch_a, cb = batches * batch_b, cc = batches * batch_c;
+      const char *ha = static_cast<const char *>(h_a) + i * chunk * batch_a;
+      const char *hb = static_cast<const char *>(h_b) + i * chunk * batch_b;
+      char *hc = static_cast<char *>(h_c) + i * chunk * batch_c;
+      if (ca) e = hipMemcpyAsync(p->lane_a[l], ha, ca, hipMemcpyHostToDevice, s);
+      if (e == hipSuccess && cb) e = hipMemcpyAsync(p->lane_b[l], hb, cb, hipMemcpyHostToDevice, s);
+      if (e == hipSuccess && p->need_copyin_c) {
+        e = hipMemcpyAsync(p->lane_c[l], hc, cc, hipMemcpyHostToDevice, s);
+      }
+      if (e != hipSuccess) break;
+      rc = ccglib_pipeline_run(lane, p->lane_a[l], p->lane_b[l], p->lane_c[l]);
+      if (rc == CCGLIB_OK) e = hipMemcpyAsync(hc, p->lane_c[l], cc, hipMemcpyDeviceToHost, s);
+    }
+    // the host Run returns with c complete (src/pipeline/Pipeline.cpp:175)
+    for (int l = 0; l < ccglib_pipeline::kHostLanes; ++l) {
+      const hipError_t es = hipStreamSynchronize(p->lane_stream[l]);
+      if (e == hipSuccess) e = es;
+    }
+    if (rc == CCGLIB_OK && e != hipSuccess) rc = fail_hip(e, "pipeline host run in chunks");
+    return rc;
+  }
+
+  void *d_a = nullptr, *d_b = nullptr, *d_c = nullptr;
+  e = hipMalloc(&d_a, bytes_a ? bytes_a : 16);
   if (e == hipSuccess) e = hipMalloc(&d_b, bytes_b ? bytes_b : 16);
   if (e == hipSuccess) e = hipMalloc(&d_c, bytes_c);
   if (e == hipSuccess && bytes_a) e = hipMemcpyAsync(d_a, h_a, bytes_a, hipMemcpyHostToDevice, p->stream);

@@ -160,7 +160,11 @@ CCGLIB_API int ccglib_packing_destroy(ccglib_packing_t packing);
  * 1-bit input is one byte per sample and is packed first; the opt variant
  * transposes A and B first. Argument order follows the reference constructor.
  * run_host copies a, b (and c when beta != 0) to the device, runs, copies c
- * back and synchronises the stream; sizes are those of the layouts above.
+ * back and returns when c is complete; sizes are those of the layouts above.
+ * Jobs of 8 MiB or more with several batches move in chunks of whole batches
+ * over two internal streams (ordered after the work already queued on the
+ * object's stream), so that with page-locked host buffers the copies in, the
+ * kernels and the copies out overlap; the result is the same either way.
  * ---------------------------------------------------------------------- */
 CCGLIB_API int ccglib_pipeline_create(
     ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,

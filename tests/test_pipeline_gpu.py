@@ -146,6 +146,74 @@ def interleaved(q, B, rows, K):
     return np.ascontiguousarray(q.reshape(B, 2, rows, K).transpose(0, 2, 3, 1)).reshape(-1)
 
 
+def _host_buffer(a, pinned):
+    """A host copy of `a` as a torch tensor (page-locked if asked) and its numpy view."""
+    t = torch.empty(a.nbytes, dtype=torch.uint8, pin_memory=pinned)
+    v = t.numpy().view(a.dtype)
+    v[:] = a.reshape(-1)
+    return t, v
+
+
+@pytest.mark.parametrize("pinned", [False, True])
+@pytest.mark.parametrize("B,M,N,K,axis,beta,chunk_bytes", [
+    (6, 256, 1024, 128, PLANAR, 0.5 - 0.25j, None),      # default size: 2 chunks of 3 batches
+    (8, 256, 512, 256, INTERLEAVED, 0, 1 << 20),         # 8 chunks of 1: every lane used again
+    (7, 200, 1000, 104, INTERLEAVED, 0, 5 << 20)])       # 2.1 MB a batch: chunks of 2, 2, 2 and 1
+def test_pipeline_host_run_in_chunks(pinned, B, M, N, K, axis, beta, chunk_bytes, monkeypatch):
+    """Host-pointer Run of a problem that takes the batch-chunked path over several
+    streams: equal, bit for bit, to the device Run of the same object, and within the
+    float bounds of the oracle."""
+    if chunk_bytes:
+        monkeypatch.setenv("CCGLIB_AMD_HOST_CHUNK_BYTES", str(chunk_bytes))
+    alpha = 1.0 if beta == 0 else 2 - 1j
+    rng = np.random.default_rng(11)
+    qa = quantize(rng.uniform(-2, 2, B * 2 * M * K), VT.float16)
+    qb = quantize(rng.uniform(-2, 2, B * 2 * N * K), VT.float16)
+    c_in = rng.uniform(-10, 10, B * 2 * M * N).astype(np.float32)
+    a_in = interleaved(qa, B, M, K) if axis == INTERLEAVED else qa
+    b_in = interleaved(qb, B, N, K) if axis == INTERLEAVED else qb
+    p = cc.Pipeline(B, M, N, K, 0, stream(), axis, PLANAR, ROW, COL, ROW, VT.float16, VT.float32,
+                    cc.Variant.opt, alpha, beta)
+    d_a, d_b, d_c = to_device(a_in), to_device(b_in), to_device(c_in)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    from_device = to_host(d_c, np.float32)
+    for _ in range(2):   # the second call re-uses the lanes
+        ta, ha = _host_buffer(a_in, pinned)
+        tb, hb = _host_buffer(b_in, pinned)
+        tc, hc = _host_buffer(c_in, pinned)
+        p.RunHost(ha.ctypes.data, hb.ctypes.data, hc.ctypes.data)
+        assert np.array_equal(hc, from_device)
+    want = orc.gemm(qa, qb, M, N, K, orc.FLOAT16, orc.FLOAT32, orc.ROW_MAJOR, alpha, beta, c_in)
+    w64 = orc.gemm_float64(qa, qb, M, N, K, orc.FLOAT16)
+    c4 = c_in.reshape(B, 2, M, N).astype(np.float64)
+    w = (w64[:, 0] + 1j * w64[:, 1]) * alpha + beta * (c4[:, 0] + 1j * c4[:, 1])
+    check_float(hc.reshape(want.shape), want, np.stack([w.real, w.imag], 1), VT.float16, VT.float32)
+
+
+@pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
+def test_pipeline_int1_host_run(axis):
+    """1-bit host Run: planar input goes through the chunked path (2 chunks of 2 batches:
+    13 MiB in all), interleaved input (packed over the whole buffer) in one piece."""
+    B, M, N, K = 4, 128, 256, 4096
+    rng = np.random.default_rng(12)
+    a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8)
+    c = rng.integers(-1000, 1000, B * 2 * M * N).astype(np.int32)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), axis, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                    cc.Variant.opt, 1.0, 1.0)
+    d_a, d_b, d_c = to_device(a_bits), to_device(b_bits), to_device(c)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = c.copy()
+    p.RunHost(a_bits.ctypes.data, b_bits.ctypes.data, got.ctypes.data)
+    assert np.array_equal(got, to_host(d_c, np.int32))
+    if axis == PLANAR:
+        want = orc.gemm(orc.pack_bits(a_bits), orc.pack_bits(b_bits), M, N, K, orc.INT1, orc.INT32,
+                        orc.ROW_MAJOR, 1.0, 1.0, c)
+        assert np.array_equal(got.reshape(want.shape), want)
+
+
 @pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.float16, VT.float16),
                                       (VT.bfloat16, VT.float32), (VT.float8e4m3, VT.float32),
                                       (VT.float8e5m2, VT.float32)])
