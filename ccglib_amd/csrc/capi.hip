@@ -107,6 +107,11 @@ struct ccglib_gemm {
   // (null: the popcount kernel runs instead)
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // Basic variant with rows that are not whole 16-byte chunks (odd K): A and B
+  // are first copied into the tiled layout (A at the start of `workspace`, B at
+  // retile_b_offset) and the kernel of the opt variant runs on the copies.
+  bool retile = false;
+  size_t retile_b_offset = 0;
 };
 
 struct ccglib_transpose {
@@ -295,6 +300,28 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
       }
     }
   }
+  const size_t eb = (size_t)bits_of(type_in) / 8;
+  const char *retile_env = std::getenv("CCGLIB_AMD_BASIC_RETILE");
+  if (type_in != kInt1 && variant == kBasic && B && M && N && K && (K * eb) % 16 != 0 &&
+      !(retile_env && std::strcmp(retile_env, "0") == 0)) {
+    // Rows that direct-to-LDS copies cannot fetch in whole chunks. Re-tiling them
+    // costs two bandwidth-bound passes and a copy of A and B; the kernel for the
+    // tiled layout then runs several times faster than the one that loads ragged
+    // rows through registers. Without the memory that kernel is used.
+    const size_t kc = (size_t)k_per_tile(type_in);
+    const size_t kp = ceil_div(K, kc) * kc;
+    const size_t bytes_a = B * 2 * ceil_div(M, kTileRows) * kTileRows * kp * eb;
+    const size_t bytes_b = B * 2 * ceil_div(N, kTileRows) * kTileRows * kp * eb;
+    DeviceGuard guard(device);
+    if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes_a + bytes_b) == hipSuccess) {
+      g->workspace_bytes = bytes_a + bytes_b;
+      g->retile = true;
+      g->retile_b_offset = bytes_a;
+    } else {
+      g->workspace = nullptr;
+      (void)hipGetLastError();
+    }
+  }
   *gemm = g;
   return CCGLIB_OK;
 }
@@ -314,6 +341,29 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   }
   DeviceGuard guard(g->device);
   HIP_TRY(guard.status());
+  if (g->retile) {
+    TransposeParams t;
+    t.batch = g->B;
+    t.n = g->K;
+    t.m_chunk = kTileRows;
+    t.n_chunk = (size_t)k_per_tile(g->type_in);
+    t.elem_bytes = bits_of(g->type_in) / 8;
+    t.interleaved = 0;
+    char *tiled_a = static_cast<char *>(g->workspace), *tiled_b = tiled_a + g->retile_b_offset;
+    t.in = d_a;
+    t.out = tiled_a;
+    t.m = g->M;
+    hipError_t et = launch_transpose(t, g->stream);
+    t.in = d_b;
+    t.out = tiled_b;
+    t.m = g->N;
+    if (et == hipSuccess) et = launch_transpose(t, g->stream);
+    if (et != hipSuccess) return fail_hip(et, "re-tiling of ragged GEMM operands");
+    fill_gemm_params(g, tiled_a, tiled_b, d_c, &p);
+    p.variant = kOpt;
+    p.workspace = nullptr;
+    p.workspace_bytes = 0;
+  }
   const hipError_t e = (g->type_in == kInt1) ? launch_gemm_int1(p, g->stream)
                                               : launch_gemm_mfma(p, g->stream);
   if (e != hipSuccess) return fail_hip(e, "GEMM kernel launch");

@@ -9,6 +9,9 @@
 namespace ccglib_amd {
 
 typedef int int4_t __attribute__((ext_vector_type(4)));
+// 16 bytes at an address that is aligned to the element size only: one wide
+// load (global memory takes any alignment on this target).
+typedef int4_t int4_unaligned_t __attribute__((aligned(1)));
 
 enum Loader { kLoadTiled = 0, kLoadPlanarVec = 1, kLoadPlanarElem = 2, kLoadInterleavedVec = 3 };
 
@@ -58,6 +61,8 @@ __device__ __forceinline__ int4_t load_chunk(const OperandView &op, unsigned kt,
       int4_t v = zero;
       if (grow >= op.rows || kb >= k_bytes) return v;
       const char *p = op.base + ((size_t)plane * op.rows + grow) * k_bytes + kb;
+      if (kb + 16 <= k_bytes) return *reinterpret_cast<const int4_unaligned_t *>(p);
+      // the chunk that holds the end of the row, element by element
       if constexpr (EB == 2) {
         const unsigned short *q = reinterpret_cast<const unsigned short *>(p);
 #pragma unroll

@@ -47,13 +47,59 @@ __device__ __forceinline__ void deinterleave(uint4_t a, uint4_t b, uint4_t &re, 
   }
 }
 
+// 16 bytes at an address that is aligned to the element size only (global
+// memory takes any alignment on this target).
+typedef uint4_t uint4_unaligned_t __attribute__((aligned(1)));
+
+template <int EB> struct ElementOf;
+template <> struct ElementOf<1> { typedef unsigned char type; };
+template <> struct ElementOf<2> { typedef unsigned short type; };
+template <> struct ElementOf<4> { typedef unsigned type; };
+
+// The output vector of elements n0 .. n0 + 16/EB - 1 of one input row that ends
+// at element n (n0 < n): whole vectors with wide loads from wherever they lie,
+// the vector that holds the end of the row element by element, zero beyond.
+// p points at element n0 (planar) or at pair n0 (interleaved).
+template <int EB, bool INTERLEAVED>
+__device__ __forceinline__ void load_ragged(const char *p, size_t plane_stride_bytes, size_t n0,
+                                            size_t n, uint4_t &re, uint4_t &im) {
+  constexpr int V = 16 / EB;
+  typedef typename ElementOf<EB>::type T;
+  if (n0 + V <= n) {
+    if constexpr (!INTERLEAVED) {
+      re = *reinterpret_cast<const uint4_unaligned_t *>(p);
+      im = *reinterpret_cast<const uint4_unaligned_t *>(p + plane_stride_bytes);
+    } else {
+      const uint4_t x = *reinterpret_cast<const uint4_unaligned_t *>(p);
+      const uint4_t y = *reinterpret_cast<const uint4_unaligned_t *>(p + 16);
+      deinterleave<EB>(x, y, re, im);
+    }
+    return;
+  }
+  struct Vec { T e[V]; };
+  Vec r = {}, i = {};
+  const T *q = reinterpret_cast<const T *>(p);
+  const T *qi = reinterpret_cast<const T *>(p + plane_stride_bytes);
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    if (n0 + e < n) {
+      r.e[e] = INTERLEAVED ? q[2 * e] : q[e];
+      i.e[e] = INTERLEAVED ? q[2 * e + 1] : qi[e];
+    }
+  }
+  re = __builtin_bit_cast(uint4_t, r);
+  im = __builtin_bit_cast(uint4_t, i);
+}
+
 constexpr int kRowsPerThread = 4;
 constexpr int kVecsPerBlockRow = 16;   // 256 bytes of a row per block
 constexpr int kRowsPerBlock = 16 * kRowsPerThread;
 
 // grid: (ceil(n_vecs_padded / 16), ceil(Mp / 64), B); block: 256 threads as
 // 16 vectors x 16 rows, each thread doing rows r, r+16, r+32, r+48.
-template <int EB, bool INTERLEAVED>
+// RAGGED: input rows of any length at any element-aligned address (the output
+// tiles still hold whole vectors per row).
+template <int EB, bool INTERLEAVED, bool RAGGED>
 __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
   constexpr int V = 16 / EB;  // elements per vector
   const size_t nvec = (size_t)blockIdx.x * kVecsPerBlockRow + (threadIdx.x & 15);
@@ -62,7 +108,7 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
   const size_t m_padded = a.m_tiles * a.m_chunk;
   if (nvec >= a.n_vecs_padded) return;
   const size_t n0 = nvec * V;
-  const bool n_ok = n0 < a.n;  // rows are whole vectors: inside or outside
+  const bool n_ok = n0 < a.n;  // (not RAGGED: rows are whole vectors, inside or outside)
   const size_t nt = nvec / a.vecs_per_tile_row, v = nvec % a.vecs_per_tile_row;
   const size_t plane_bytes = a.m_chunk * a.n_chunk * EB;
 
@@ -73,7 +119,11 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
     re[i] = uint4_t{0, 0, 0, 0};
     im[i] = uint4_t{0, 0, 0, 0};
     if (m < a.m && n_ok) {
-      if constexpr (!INTERLEAVED) {
+      if constexpr (RAGGED) {
+        const char *p = INTERLEAVED ? a.in + ((b * a.m + m) * a.n + n0) * 2 * EB
+                                    : a.in + (((b * 2) * a.m + m) * a.n + n0) * EB;
+        load_ragged<EB, INTERLEAVED>(p, a.m * a.n * EB, n0, a.n, re[i], im[i]);
+      } else if constexpr (!INTERLEAVED) {
         const char *p = a.in + (((b * 2) * a.m + m) * a.n + n0) * EB;
         re[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
         im[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p + a.m * a.n * EB));
@@ -142,18 +192,28 @@ hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
   constexpr size_t V = 16 / EB;
   const size_t m_padded = a.m_tiles * a.m_chunk, n_padded = a.n_tiles * a.n_chunk;
   if (p.batch == 0 || m_padded == 0 || n_padded == 0) return hipSuccess;
-  const bool vec_ok = (p.n_chunk % V == 0) && (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0) &&
-                      ((uintptr_t)p.out % 16 == 0) && p.batch <= 65535 &&
-                      ceil_div(m_padded, kRowsPerBlock) <= 65535;
-  if (vec_ok) {
+  // whole vectors per output tile row; the input may be ragged
+  const bool out_vec_ok = (p.n_chunk % V == 0) && ((uintptr_t)p.out % 16 == 0) &&
+                          ((uintptr_t)p.in % EB == 0) && p.batch <= 65535 &&
+                          ceil_div(m_padded, kRowsPerBlock) <= 65535;
+  const bool in_vec_ok = (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0);
+  if (out_vec_ok) {
     a.n_vecs_padded = n_padded / V;
     a.vecs_per_tile_row = p.n_chunk / V;
     const dim3 grid((unsigned)ceil_div(a.n_vecs_padded, kVecsPerBlockRow),
                     (unsigned)ceil_div(m_padded, kRowsPerBlock), (unsigned)p.batch);
     if (p.interleaved) {
-      hipLaunchKernelGGL((transpose_vec<EB, true>), grid, dim3(256), 0, stream, a);
+      if (in_vec_ok) {
+        hipLaunchKernelGGL((transpose_vec<EB, true, false>), grid, dim3(256), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL((transpose_vec<EB, true, true>), grid, dim3(256), 0, stream, a);
+      }
     } else {
-      hipLaunchKernelGGL((transpose_vec<EB, false>), grid, dim3(256), 0, stream, a);
+      if (in_vec_ok) {
+        hipLaunchKernelGGL((transpose_vec<EB, false, false>), grid, dim3(256), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL((transpose_vec<EB, false, true>), grid, dim3(256), 0, stream, a);
+      }
     }
   } else {
     a.n_vecs_padded = 0;

@@ -144,17 +144,29 @@ def test_opt(tin, tout, M, N, K, c_order, c_axis):
     float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=True, seed=5)
 
 
+def basic_variant(variant, monkeypatch):
+    """The basic variant copies operands with ragged rows (K·size not a multiple of 16
+    bytes) into the tiled layout first; "basic_no_retile" switches that off, which
+    leaves the kernel that loads ragged rows itself."""
+    if variant == "basic_no_retile":
+        monkeypatch.setenv("CCGLIB_AMD_BASIC_RETILE", "0")
+        return cc.Variant.basic
+    return variant
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000),
                                    (257, 129, 72), (130, 2, 2049)])
-@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
-def test_odd_shapes_fp16(M, N, K, variant):
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt, "basic_no_retile"])
+def test_odd_shapes_fp16(M, N, K, variant, monkeypatch):
+    variant = basic_variant(variant, monkeypatch)
     float_case(2, M, N, K, VT.float16, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000), (257, 129, 72)])
-@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
-def test_odd_shapes_fp32(M, N, K, variant):
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt, "basic_no_retile"])
+def test_odd_shapes_fp32(M, N, K, variant, monkeypatch):
     # K not a multiple of the 16 values of a tile row, rows that are not whole 16-byte chunks
+    variant = basic_variant(variant, monkeypatch)
     float_case(2, M, N, K, VT.float32, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
 
 
@@ -166,9 +178,12 @@ def test_fp32_alpha_beta_and_many_tiles():
 
 @pytest.mark.parametrize("tin", [VT.float8e4m3, VT.float8e5m2])
 @pytest.mark.parametrize("K", [1, 63, 64, 65, 128, 192, 200])
-def test_fp8_k_tails(tin, K):
+def test_fp8_k_tails(tin, K, monkeypatch):
     # an MFMA consumes two 64-value K tiles; odd tile counts and ragged tails
     float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=K)
+    with monkeypatch.context() as m:
+        m.setenv("CCGLIB_AMD_BASIC_RETILE", "0")
+        float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=K)
     float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.opt, PLANAR, COL, seed=K + 1)
 
 

@@ -14,7 +14,7 @@ PLANAR, INTERLEAVED = cc.ComplexAxisLocation.complex_planar, cc.ComplexAxisLocat
 NP = {8: np.uint8, 16: np.uint16, 32: np.uint32, 1: np.uint32}
 
 
-def run_case(B, M, N, Mc, Nc, bits, axis, seed=0, host=False):
+def run_case(B, M, N, Mc, Nc, bits, axis, seed=0, host=False, skew=0):
     rng = np.random.default_rng(seed)
     dt = NP[bits]
     nw = N // 32 if bits == 1 else N
@@ -25,8 +25,9 @@ def run_case(B, M, N, Mc, Nc, bits, axis, seed=0, host=False):
     if host:
         t.RunHost(x.ctypes.data, d_out.data_ptr())
     else:
-        d_in = to_device(x)
-        t.Run(d_in.data_ptr(), d_out.data_ptr())
+        # skew: the input starts `skew` elements past a 16-byte boundary
+        d_in = to_device(np.concatenate([np.zeros(skew, dtype=dt), x]))
+        t.Run(d_in.data_ptr() + skew * dt().itemsize, d_out.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(to_host(d_out, dt), want)
 
@@ -52,6 +53,15 @@ def test_gemm_chunks(axis, bits, kc, M, N):
     # chunk sizes the GEMM asks for; shapes with ragged rows, ragged columns and
     # rows that are not whole 16-byte vectors (scalar kernel)
     run_case(3, M, N, 128, kc, bits, axis, seed=M + N)
+
+
+@pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
+@pytest.mark.parametrize("bits,kc", [(16, 32), (8, 64), (32, 16)])
+@pytest.mark.parametrize("M,N,skew", [(130, 1001, 0), (64, 257, 3), (200, 96, 1), (3, 15, 5), (97, 8001, 0)])
+def test_ragged_rows(axis, bits, kc, M, N, skew):
+    # rows of any length at any element-aligned address: whole vectors are moved
+    # with wide loads wherever they lie, the end of a row element by element
+    run_case(2, M, N, 128, kc, bits, axis, seed=N + skew, skew=skew)
 
 
 @pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
