@@ -716,6 +716,47 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
   }
 }
 
+// The same for interleaved fp32 C: 16 rows of 32 (re, im) pairs at a time (half
+// the width of the wave tile, again 256 bytes per row) go through the patch.
+template <int TX, int TY>
+__device__ __forceinline__ void store_wave_tile_staged_il(const KernelArgs &args, unsigned b,
+                                                          unsigned x_wave, unsigned y_wave, int lane,
+                                                          char *patch, float4_t (&acc_re)[TY][TX],
+                                                          float4_t (&acc_im)[TY][TX]) {
+  static_assert(TX == 4, "two halves of 32 columns");
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha;
+  const float ar = args.alpha_re, ai = args.alpha_im;
+  float *cbase = reinterpret_cast<float *>(args.c) + (size_t)b * 2 * nx * ny;
+  char *wr = patch + (lane & 15) * 272 + (lane >> 4) * 32;   // [y = lane%16][pair (lane/16)*4 ..]
+  const char *rd = patch + (lane >> 4) * 272 + (lane & 15) * 16;  // [row lane/16][pairs 2 (lane%16) ..]
+  float *out = cbase + ((size_t)(y_wave + (lane >> 4)) * nx + x_wave) * 2 + (lane & 15) * 4;
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int i = 2 * h; i < 2 * h + 2; ++i) {
+        float re[4], im[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float r0 = acc_re[j][i][e], i0 = acc_im[j][i][e];
+          re[e] = have_alpha ? ar * r0 - ai * i0 : r0;
+          im[e] = have_alpha ? ai * r0 + ar * i0 : i0;
+        }
+        char *w = wr + (i - 2 * h) * 128;
+        *reinterpret_cast<float4_t *>(w) = float4_t{re[0], im[0], re[1], im[1]};
+        *reinterpret_cast<float4_t *>(w + 16) = float4_t{re[2], im[2], re[3], im[3]};
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float4_t v = *reinterpret_cast<const float4_t *>(rd + r * 4 * 272);
+        *reinterpret_cast<float4_t *>(out + ((size_t)(j * 16 + r * 4) * nx + h * 32) * 2) = v;
+      }
+    }
+  }
+}
+
 // The same for the 32-row MFMA layout: one 32 x 32 tile at a time goes through
 // a patch of 32 rows of 144 bytes (128 + 16 of padding), and every store
 // instruction writes eight whole 128-byte row segments.
@@ -1093,9 +1134,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int xil_off[2] = {(wx * WX) * 128 + il_off[0], (wx * WX) * 128 + il_off[1]};
   const int yil_off[2] = {X_BYTES + (wy * WY) * 128 + il_off[0],
                           X_BYTES + (wy * WY) * 128 + il_off[1]};
-  // wide stores through LDS: planar C, no beta term, vector-aligned rows
-  const bool staged_ok = !args.c_interleaved && !args.have_beta && args.c_vector_ok &&
-                         (args.nx % 4 == 0);
+  // wide stores through LDS: no beta term, vector-aligned rows (interleaved C
+  // only with the 16-row layout)
+  const bool staged_ok = (MS == 16 || !args.c_interleaved) && !args.have_beta &&
+                         args.c_vector_ok && (args.nx % 4 == 0);
 
   // ---- pipeline ----------------------------------------------------------
   point_at(load_tile);
@@ -1188,9 +1230,12 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
-          store_wave_tile_staged<TX, TY>(args, tc.b, x_wave, y_wave, lane,
-                                         lds + free_slot * SLOT_BYTES + wave * kStagePatchBytes,
-                                         acc_re, acc_im);
+          char *patch = lds + free_slot * SLOT_BYTES + wave * kStagePatchBytes;
+          if (args.c_interleaved) {
+            store_wave_tile_staged_il<TX, TY>(args, tc.b, x_wave, y_wave, lane, patch, acc_re, acc_im);
+          } else {
+            store_wave_tile_staged<TX, TY>(args, tc.b, x_wave, y_wave, lane, patch, acc_re, acc_im);
+          }
           staged = true;
         }
       }

@@ -170,6 +170,16 @@ def test_odd_shapes_fp32(M, N, K, variant, monkeypatch):
     float_case(2, M, N, K, VT.float32, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
 
 
+@pytest.mark.parametrize("c_order", [ROW, COL])
+@pytest.mark.parametrize("tin", [VT.float16, VT.bfloat16, VT.float8e4m3])
+def test_interleaved_c_alpha_only(tin, c_order):
+    # beta = 0 and aligned rows: wave tiles inside C go through the LDS-staged wide
+    # stores, the ragged right and bottom edges (M = 300, N = 328) through the direct ones
+    float_case(3, 300, 328, 96, tin, VT.float32, cc.Variant.opt, INTERLEAVED, c_order,
+               alpha=0.75 - 0.5j, seed=21)
+    float_case(2, 256, 512, 64, tin, VT.float32, cc.Variant.opt, INTERLEAVED, c_order, seed=22)
+
+
 def test_fp32_alpha_beta_and_many_tiles():
     float_case(3, 256, 320, 96, VT.float32, VT.float32, cc.Variant.opt, INTERLEAVED, COL,
                alpha=0.75 - 0.5j, beta=0.5 - 0.25j)
