@@ -492,6 +492,85 @@ __device__ __forceinline__ void mma_step_interleaved(const char *slot, const int
   }
 }
 
+// The interleaved step for 16-bit input and a 4 x 4 wave tile with the LDS reads
+// placed by hand (see mma_step_ordered): a wave reads what its first MFMAs
+// need, fetches the raw Y fragment of the next tile row while the current one
+// is multiplied, and the X fragments of the slot's second half during the
+// first half's last rows.
+template <int DT, int BX, int BY, typename Mid>
+__device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, const int (&x_off)[2],
+                                                             const int (&y_off)[2],
+                                                             float4_t (&acc_re)[4][4],
+                                                             float4_t (&acc_im)[4][4], Mid &&mid) {
+  static_assert(DtypeTraits<DT>::kTilesPerMfma == 1 && DtypeTraits<DT>::kElemBytes == 2,
+                "16-bit input");
+  auto rd = [&](int off) {
+    Fragment<DT> f;
+    f.v[0] = *reinterpret_cast<const int4_t *>(slot + off);
+    return f;
+  };
+  // (yr, -yi, ...) and (yi, yr, ...) of a raw fragment (yr, yi, ...)
+  auto flip = [](const Fragment<DT> &raw) {
+    Fragment<DT> f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) f.v[0][w] = (int)((unsigned)raw.v[0][w] ^ 0x80000000u);
+    return f;
+  };
+  auto swap = [](const Fragment<DT> &raw) {
+    Fragment<DT> f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const unsigned v = (unsigned)raw.v[0][w];
+      f.v[0][w] = (int)__builtin_amdgcn_alignbit(v, v, 16);
+    }
+    return f;
+  };
+  constexpr int ROW16 = 16 * 128;
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+  Fragment<DT> xa[4], xb[4], raw, y1, y2;
+  raw = rd(y_off[0]);
+  xa[0] = rd(x_off[0]);
+  xa[1] = rd(x_off[0] + ROW16);
+  xa[2] = rd(x_off[0] + 2 * ROW16);
+  CCGLIB_PIN;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    Fragment<DT>(&x)[4] = h == 0 ? xa : xb;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      y1 = flip(raw);
+      y2 = swap(raw);
+      CCGLIB_PIN;
+      acc_re[j][0] = mfma<DT>(x[0], y1, acc_re[j][0]);
+      if (h == 0 && j == 0) xa[3] = rd(x_off[0] + 3 * ROW16);
+      // the raw Y fragment of the next row (of this half, then of the other)
+      if (j < 3) {
+        raw = rd(y_off[h] + (j + 1) * ROW16);
+      } else if (h == 0) {
+        raw = rd(y_off[1]);
+      }
+      CCGLIB_PIN;
+      acc_im[j][0] = mfma<DT>(x[0], y2, acc_im[j][0]);
+      if (h == 0 && j >= 2) xb[2 * (j - 2)] = rd(x_off[1] + 2 * (j - 2) * ROW16);
+      CCGLIB_PIN;
+      acc_re[j][1] = mfma<DT>(x[1], y1, acc_re[j][1]);
+      if (h == 0 && j >= 2) xb[2 * (j - 2) + 1] = rd(x_off[1] + (2 * (j - 2) + 1) * ROW16);
+      CCGLIB_PIN;
+      acc_im[j][1] = mfma<DT>(x[1], y2, acc_im[j][1]);
+      acc_re[j][2] = mfma<DT>(x[2], y1, acc_re[j][2]);
+      acc_im[j][2] = mfma<DT>(x[2], y2, acc_im[j][2]);
+      acc_re[j][3] = mfma<DT>(x[3], y1, acc_re[j][3]);
+      acc_im[j][3] = mfma<DT>(x[3], y2, acc_im[j][3]);
+      CCGLIB_PIN;
+      if (h == 0 && j == 0) {
+        mid();
+        CCGLIB_PIN;
+      }
+    }
+  }
+#undef CCGLIB_PIN
+}
+
 // Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
 // store, piece by piece (four consecutive elements of the contiguous C axis).
 template <int TOUT, int TX, int TY, int MS = 16, typename Acc>
@@ -1191,7 +1270,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           for (int u = 0; u < KPI; ++u) issue_next(refill + u);
         }
       };
-      if constexpr (IL) {
+      if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
+        mma_step_interleaved_ordered<DT, BX, BY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
+                                                 acc_im, refill_slots);
+      } else if constexpr (IL) {
         mma_step_interleaved<DT, BX, BY, TX, TY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
                                                  acc_im, refill_slots);
       } else {

@@ -32,6 +32,7 @@ struct Config {
   const char *name;
   LaunchFn launch;
   int type_in, type_out;
+  int layout = kLoadTiled;   // operand layout the configuration reads
 };
 
 // name: type, block BX x BY, wave WX x WY, ring slots, MFMA rows
@@ -45,6 +46,11 @@ static const std::vector<Config> kConfigs = {
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"fp8 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat8e4m3, kFloat32},
     {"fp4 256x128 w64x64 s3 m32", launch_dtl<kFp4Sign, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFp4Sign, kInt32},
+    // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
+    {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
+    {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
+    {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
+    {"fp8 interleaved 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec, 16>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
 };
 
 static double peak_of(int type) {
@@ -89,7 +95,7 @@ int main(int argc, char **argv) {
   hipEvent_t e0, e1;
   CHECK(hipEventCreate(&e0));
   CHECK(hipEventCreate(&e1));
-  std::printf("%-32s %10s %12s %10s   (B=%u M=%u N=%u K=%u%s)\n", "configuration", "ms", "TFLOP/s", "of peak", B, M, N, K,
+  std::printf("%-40s %10s %12s %10s   (B=%u M=%u N=%u K=%u%s)\n", "configuration", "ms", "TFLOP/s", "of peak", B, M, N, K,
               std::getenv("ZERO") ? ", zero operands" : "");
   for (const Config &c : kConfigs) {
     if (filter && !std::strstr(c.name, filter)) continue;
@@ -99,22 +105,24 @@ int main(int argc, char **argv) {
     p.nx = N;
     p.ny = M;
     p.k = K;
-    p.k_tiles = (K + kpt - 1) / kpt;
+    p.k_tiles = ((c.layout == kLoadInterleavedVec ? 2 * K : K) + kpt - 1) / kpt;
     p.x_tiles = (N + kTileRows - 1) / kTileRows;
     p.y_tiles = (M + kTileRows - 1) / kTileRows;
     p.type_in = c.type_in;
     p.type_out = c.type_out;
-    p.variant = kOpt;
+    p.variant = c.layout == kLoadPlanarVec ? kBasic : kOpt;
     p.c_interleaved = 0;
-    p.input_interleaved = 0;
+    p.input_interleaved = c.layout == kLoadInterleavedVec;
     p.alpha_re = 1;
     p.alpha_im = 0;
     p.beta_re = 0;
     p.beta_im = 0;
     p.have_alpha = 0;
     p.have_beta = 0;
-    const size_t x_bytes = (size_t)B * p.x_tiles * p.k_tiles * kTileBytes;
-    const size_t y_bytes = (size_t)B * p.y_tiles * p.k_tiles * kTileBytes;
+    // whole tiles: at least as large as the planar and interleaved layouts
+    const unsigned k_tiles_planar = (K + kpt - 1) / kpt;
+    const size_t x_bytes = (size_t)B * p.x_tiles * k_tiles_planar * kTileBytes;
+    const size_t y_bytes = (size_t)B * p.y_tiles * k_tiles_planar * kTileBytes;
     const size_t c_bytes = (size_t)B * 2 * M * N * 4;
     void *dx, *dy, *dc;
     CHECK(hipMalloc(&dx, x_bytes));
@@ -153,7 +161,7 @@ int main(int argc, char **argv) {
     CHECK(hipEventElapsedTime(&best, e0, e1));
     best /= iters;
     const double tflops = 8.0 * B * M * N * K / (best * 1e-3) / 1e12;
-    std::printf("%-32s %10.4f %12.1f %9.1f%%\n", c.name, best, tflops, 100 * tflops / peak_of(c.type_in));
+    std::printf("%-40s %10.4f %12.1f %9.1f%%\n", c.name, best, tflops, 100 * tflops / peak_of(c.type_in));
     std::fflush(stdout);
     CHECK(hipFree(dx));
     CHECK(hipFree(dy));
