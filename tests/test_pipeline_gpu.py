@@ -246,6 +246,26 @@ def test_pipeline_interleaved_input(tin, tout, K, variant):
     check_float(got, dequantize(want, tout), np.stack([w.real, w.imag], 1), tin, tout)
 
 
+@pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
+def test_pipeline_interleaved_input_large_c(tin):
+    # With M N / (M + N) above about 2000 the opt pipeline transposes interleaved input
+    # into tiles instead of reading the rows in place (the GEMM then runs enough faster
+    # to pay for the two transposes); same numbers either way.
+    B, M, N, K = 1, 4096, 4096, 64
+    rng = np.random.default_rng(31)
+    qa = quantize(rng.uniform(-1, 1, B * 2 * M * K), tin)
+    qb = quantize(rng.uniform(-1, 1, B * 2 * N * K), tin)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, tin, VT.float32,
+                    cc.Variant.opt)
+    d_a, d_b = to_device(interleaved(qa, B, M, K)), to_device(interleaved(qb, B, N, K))
+    d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, np.float32).reshape(B, 2, M, N)
+    want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[tin], orc.FLOAT32)
+    check_float(got, want, orc.gemm_float64(qa, qb, M, N, K, ORC_TYPE[tin]), tin, VT.float32)
+
+
 def test_pipeline_basic_rejects_interleaved_output():
     with pytest.raises(RuntimeError, match="complex-interleaved output is not supported in basic variant"):
         cc.Pipeline(1, 16, 16, 16, 0, stream(), PLANAR, INTERLEAVED, ROW, COL, ROW, VT.float16,
