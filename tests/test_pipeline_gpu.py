@@ -248,7 +248,7 @@ def test_pipeline_interleaved_input(tin, tout, K, variant):
 
 @pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
 def test_pipeline_interleaved_input_large_c(tin):
-    # With M N / (M + N) above about 2000 the opt pipeline transposes interleaved input
+    # With M N / (M + N) above about 2000 (330 for 8-bit input) the opt pipeline transposes interleaved input
     # into tiles instead of reading the rows in place (the GEMM then runs enough faster
     # to pay for the two transposes); same numbers either way.
     B, M, N, K = 1, 4096, 4096, 64
