@@ -649,7 +649,13 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   const bool fused = !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&
                      (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2000.0 : 330.0));
-  const bool transposing = (variant == kOpt) && !fused;   // :53
+  // The reference transposes for the opt variant only (:53) and hands interleaved
+  // input of the basic variant to a kernel that reads it as planar. Here such
+  // input is always de-interleaved: in the GEMM's loader (fused) or, where that
+  // cannot take the rows, by the transposes, with the tiled kernel behind them.
+  const bool basic_needs_tiles = !packing && variant == kBasic &&
+                                 input_complex_axis_location == kInterleaved && !fused;
+  const bool transposing = ((variant == kOpt) && !fused) || basic_needs_tiles;
   // Packing already moves all real samples in front of all imaginary ones
   // (over the whole buffer), so what follows it sees planar data.
   const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
@@ -710,7 +716,8 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
       }
     }
     rc = ccglib_gemm_create(&p->gemm, B, M, N, K, device, stream, input_type, output_type,
-                            fused ? (int)kOpt : variant, output_complex_axis_location,
+                            (fused || basic_needs_tiles) ? (int)kOpt : variant,
+                            output_complex_axis_location,
                             c_mem_order, a_mem_order, b_mem_order, alpha_re, alpha_im, beta_re,
                             beta_im);  // :102-105
     if (rc == CCGLIB_OK) p->gemm->input_interleaved = fused;
