@@ -492,11 +492,14 @@ __device__ __forceinline__ void mma_step_interleaved(const char *slot, const int
   }
 }
 
-// The interleaved step for 16-bit input and a 4 x 4 wave tile with the LDS reads
-// placed by hand (see mma_step_ordered): a wave reads what its first MFMAs
-// need, fetches the raw Y fragment of the next tile row while the current one
-// is multiplied, and the X fragments of the slot's second half during the
-// first half's last rows.
+// The interleaved step for 16-bit input and a 4 x 4 wave tile with every LDS
+// read and every derived fragment placed by hand (see mma_step_ordered). The
+// slot is walked as eight tile rows (two halves of K x four rows of Y). The raw
+// Y fragment of a row is read two rows ahead; its two variants are computed
+// during the previous row, two instructions behind each of that row's last
+// four MFMAs, where they issue in the shadow of the matrix instruction instead
+// of holding up the next row; the X fragments of the second half are fetched
+// during rows 2 and 3.
 template <int DT, int BX, int BY, typename Mid>
 __device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, const int (&x_off)[2],
                                                              const int (&y_off)[2],
@@ -509,64 +512,78 @@ __device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, c
     f.v[0] = *reinterpret_cast<const int4_t *>(slot + off);
     return f;
   };
-  // (yr, -yi, ...) and (yi, yr, ...) of a raw fragment (yr, yi, ...)
-  auto flip = [](const Fragment<DT> &raw) {
-    Fragment<DT> f;
+  // words w0, w0 + 1 of (yr, -yi, ...) and of (yi, yr, ...) from the raw (yr, yi, ...).
+  // The empty asm statement takes the result where it is computed: without it,
+  // arithmetic whose result is first used in the next row is sunk there before
+  // the instructions are scheduled. (The arithmetic itself stays ordinary code,
+  // so the compiler keeps track of the wait states the MFMAs need.)
+  auto flip2 = [](Fragment<DT> &f, const Fragment<DT> &raw, int w0) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) f.v[0][w] = (int)((unsigned)raw.v[0][w] ^ 0x80000000u);
-    return f;
-  };
-  auto swap = [](const Fragment<DT> &raw) {
-    Fragment<DT> f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const unsigned v = (unsigned)raw.v[0][w];
-      f.v[0][w] = (int)__builtin_amdgcn_alignbit(v, v, 16);
+    for (int w = w0; w < w0 + 2; ++w) {
+      int o = (int)((unsigned)raw.v[0][w] ^ 0x80000000u);
+      asm volatile("" : "+v"(o));
+      f.v[0][w] = o;
     }
-    return f;
+  };
+  auto swap2 = [](Fragment<DT> &f, const Fragment<DT> &raw, int w0) {
+#pragma unroll
+    for (int w = w0; w < w0 + 2; ++w) {
+      const unsigned v = (unsigned)raw.v[0][w];
+      int o = (int)__builtin_amdgcn_alignbit(v, v, 16);
+      asm volatile("" : "+v"(o));
+      f.v[0][w] = o;
+    }
   };
   constexpr int ROW16 = 16 * 128;
+  auto y_row_off = [&](int r) { return y_off[r >> 2] + (r & 3) * ROW16; };
 #define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
-  Fragment<DT> xa[4], xb[4], raw, y1, y2;
-  raw = rd(y_off[0]);
+  Fragment<DT> xa[4], xb[4], raw[2], y1, y2, y1n, y2n;
+  raw[0] = rd(y_row_off(0));
   xa[0] = rd(x_off[0]);
   xa[1] = rd(x_off[0] + ROW16);
+  raw[1] = rd(y_row_off(1));
   xa[2] = rd(x_off[0] + 2 * ROW16);
   CCGLIB_PIN;
+  flip2(y1, raw[0], 0);
+  flip2(y1, raw[0], 2);
+  swap2(y2, raw[0], 0);
+  swap2(y2, raw[0], 2);
+  CCGLIB_PIN;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    Fragment<DT>(&x)[4] = h == 0 ? xa : xb;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      y1 = flip(raw);
-      y2 = swap(raw);
+  for (int r = 0; r < 8; ++r) {
+    const int j = r & 3;
+    Fragment<DT>(&x)[4] = r < 4 ? xa : xb;
+    const Fragment<DT> &next_raw = raw[(r + 1) & 1];
+    acc_re[j][0] = mfma<DT>(x[0], y1, acc_re[j][0]);
+    if (r == 0) xa[3] = rd(x_off[0] + 3 * ROW16);
+    if (r + 2 < 8) raw[r & 1] = rd(y_row_off(r + 2));   // this row's raw fragment is used up
+    CCGLIB_PIN;
+    acc_im[j][0] = mfma<DT>(x[0], y2, acc_im[j][0]);
+    if (r == 2 || r == 3) xb[2 * (r - 2)] = rd(x_off[1] + 2 * (r - 2) * ROW16);
+    CCGLIB_PIN;
+    acc_re[j][1] = mfma<DT>(x[1], y1, acc_re[j][1]);
+    if (r == 2 || r == 3) xb[2 * (r - 2) + 1] = rd(x_off[1] + (2 * (r - 2) + 1) * ROW16);
+    CCGLIB_PIN;
+    acc_im[j][1] = mfma<DT>(x[1], y2, acc_im[j][1]);
+    CCGLIB_PIN;
+    acc_re[j][2] = mfma<DT>(x[2], y1, acc_re[j][2]);
+    if (r + 1 < 8) flip2(y1n, next_raw, 0);
+    CCGLIB_PIN;
+    acc_im[j][2] = mfma<DT>(x[2], y2, acc_im[j][2]);
+    if (r + 1 < 8) flip2(y1n, next_raw, 2);
+    CCGLIB_PIN;
+    acc_re[j][3] = mfma<DT>(x[3], y1, acc_re[j][3]);
+    if (r + 1 < 8) swap2(y2n, next_raw, 0);
+    CCGLIB_PIN;
+    acc_im[j][3] = mfma<DT>(x[3], y2, acc_im[j][3]);
+    if (r + 1 < 8) swap2(y2n, next_raw, 2);
+    CCGLIB_PIN;
+    if (r == 0) {
+      mid();
       CCGLIB_PIN;
-      acc_re[j][0] = mfma<DT>(x[0], y1, acc_re[j][0]);
-      if (h == 0 && j == 0) xa[3] = rd(x_off[0] + 3 * ROW16);
-      // the raw Y fragment of the next row (of this half, then of the other)
-      if (j < 3) {
-        raw = rd(y_off[h] + (j + 1) * ROW16);
-      } else if (h == 0) {
-        raw = rd(y_off[1]);
-      }
-      CCGLIB_PIN;
-      acc_im[j][0] = mfma<DT>(x[0], y2, acc_im[j][0]);
-      if (h == 0 && j >= 2) xb[2 * (j - 2)] = rd(x_off[1] + 2 * (j - 2) * ROW16);
-      CCGLIB_PIN;
-      acc_re[j][1] = mfma<DT>(x[1], y1, acc_re[j][1]);
-      if (h == 0 && j >= 2) xb[2 * (j - 2) + 1] = rd(x_off[1] + (2 * (j - 2) + 1) * ROW16);
-      CCGLIB_PIN;
-      acc_im[j][1] = mfma<DT>(x[1], y2, acc_im[j][1]);
-      acc_re[j][2] = mfma<DT>(x[2], y1, acc_re[j][2]);
-      acc_im[j][2] = mfma<DT>(x[2], y2, acc_im[j][2]);
-      acc_re[j][3] = mfma<DT>(x[3], y1, acc_re[j][3]);
-      acc_im[j][3] = mfma<DT>(x[3], y2, acc_im[j][3]);
-      CCGLIB_PIN;
-      if (h == 0 && j == 0) {
-        mid();
-        CCGLIB_PIN;
-      }
     }
+    y1 = y1n;
+    y2 = y2n;
   }
 #undef CCGLIB_PIN
 }
