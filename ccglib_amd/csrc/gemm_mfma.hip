@@ -22,6 +22,8 @@
 //    sign of Re -= Xi*Yi is a sign-bit flip of the Yi fragment registers.
 //  * Workgroup ids are remapped so that consecutive tiles land on the same
 //    XCD (shared L2), in groups that reuse both operands.
+#include <atomic>
+
 #include "gemm_device.h"
 
 namespace ccglib_amd {
@@ -1369,11 +1371,20 @@ inline hipError_t check_grid(size_t total) {
   return total > 0x7fffffffu ? hipErrorInvalidValue : hipSuccess;
 }
 
-// LDS beyond 64 KiB has to be requested once per kernel.
-template <typename Kernel> hipError_t allow_lds(Kernel kernel, int bytes) {
+// LDS beyond 64 KiB has to be requested once per kernel and device. `done`
+// is the caller's per-kernel record (one flag per device ordinal).
+constexpr int kMaxDevices = 64;
+template <typename Kernel>
+hipError_t allow_lds(Kernel kernel, int bytes, std::atomic<bool> (&done)[kMaxDevices]) {
   if (bytes <= 64 * 1024) return hipSuccess;
-  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && done[dev].load(std::memory_order_acquire)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && tracked) done[dev].store(true, std::memory_order_release);
+  return e;
 }
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int KT, int LOADER, int WPE>
@@ -1385,8 +1396,8 @@ hipError_t launch_config(const GemmParams &p, hipStream_t stream) {
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
   auto kernel = complex_gemm_mfma<DT, TOUT, BX, BY, WX, WY, KT, LOADER, WPE>;
-  static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
-  if (lds_ok != hipSuccess) return lds_ok;
+  static std::atomic<bool> lds_allowed[kMaxDevices];
+  if (hipError_t e = allow_lds(kernel, LDS_BYTES, lds_allowed)) return e;
   hipLaunchKernelGGL(kernel, dim3((unsigned)total), dim3(NTHREADS), LDS_BYTES, stream, a);
   return hipGetLastError();
 }
@@ -1420,8 +1431,8 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
   auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS>;
-  static const hipError_t lds_ok = allow_lds(kernel, LDS_BYTES);
-  if (lds_ok != hipSuccess) return lds_ok;
+  static std::atomic<bool> lds_allowed[kMaxDevices];
+  if (hipError_t e = allow_lds(kernel, LDS_BYTES, lds_allowed)) return e;
   // persistent blocks: as many as are resident at once, each walking C tiles
   // with a stride of the grid size (a multiple of the XCD count)
   const size_t resident = (size_t)compute_units() * BLOCKS_PER_CU / kNumXcd * kNumXcd;
