@@ -198,6 +198,24 @@ __device__ __forceinline__ unsigned spread8(unsigned x) {
   return x;
 }
 
+// 32 samples -> 32 nibbles: 0x2 | bit << 3 where the sample exists, 0 where it
+// does not (bits of `word` outside `valid` are zero). Whole words, which is all
+// of them except at the end of K, skip the second spread: the kernels are close
+// to being bound by this arithmetic rather than by their stores.
+__device__ __forceinline__ uint4_t nibbles_of(unsigned word, unsigned valid) {
+  uint4_t o;
+  if (valid == 0xffffffffu) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = (spread8((word >> (8 * q)) & 0xffu) << 3) | 0x22222222u;
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o[q] = (spread8((word >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
+    }
+  }
+  return o;
+}
+
 // A thread takes word c (of four) of each of the four 128-sample K tiles that a
 // 64-byte row of the 1-bit layout spans: four 4-byte loads in flight per thread
 // (with one, the kernel is bound by the latency of its reads), and every store
@@ -243,11 +261,7 @@ __global__ __launch_bounds__(256) void expand_int1_to_fp4(const char *__restrict
     const unsigned n = first >= k ? 0u : (k - first >= 32 ? 32u : k - first);
     const unsigned valid = n == 32 ? 0xffffffffu : ((1u << n) - 1u);
     const unsigned ws = w[s] & valid;
-    uint4_t o;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      o[q] = (spread8((ws >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
-    }
+    const uint4_t o = nibbles_of(ws, valid);
     __builtin_nontemporal_store(
         o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
                                        plane * kTilePlaneBytes + row * kTileRowBytes + 16 * c));
@@ -305,11 +319,7 @@ __global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *
       for (unsigned i = 0; i < n[s]; ++i) bits[s] |= (row_ptr[k0 + i] != 0 ? 1u : 0u) << i;
     }
     const unsigned valid = n[s] == 32 ? 0xffffffffu : ((1u << n[s]) - 1u);
-    uint4_t o;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      o[q] = (spread8((bits[s] >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
-    }
+    const uint4_t o = nibbles_of(bits[s], valid);
     __builtin_nontemporal_store(
         o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
                                        plane * kTilePlaneBytes + row_in_tile * kTileRowBytes + 16 * c));
