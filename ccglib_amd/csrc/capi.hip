@@ -107,6 +107,9 @@ struct ccglib_gemm {
   // (null: the popcount kernel runs instead)
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // 1-bit GEMM with a workspace: a second stream on which the expansion of later
+  // batches runs while earlier ones are multiplied (null members: not in use)
+  GemmAux aux;
   // Basic variant with rows that are not whole 16-byte chunks (odd K): A and B
   // are first copied into the tiled layout (A at the start of `workspace`, B at
   // retile_b_offset) and the kernel of the opt variant runs on the copies.
@@ -161,6 +164,17 @@ struct ccglib_pipeline {
 
 namespace {
 
+void release_aux(GemmAux *aux) {
+  for (int i = 0; i < GemmAux::kMaxJoins; ++i) {
+    if (aux->join[i]) (void)hipEventDestroy(aux->join[i]);
+    aux->join[i] = nullptr;
+  }
+  if (aux->fork) (void)hipEventDestroy(aux->fork);
+  if (aux->stream) (void)hipStreamDestroy(aux->stream);
+  aux->fork = nullptr;
+  aux->stream = nullptr;
+}
+
 // Launch parameters of a GEMM object for the given buffers.
 void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, void *d_c,
                       GemmParams *out) {
@@ -199,6 +213,7 @@ void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, vo
   p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
   p.workspace = g->workspace;
   p.workspace_bytes = g->workspace_bytes;
+  p.aux = g->aux.stream ? &g->aux : nullptr;
 }
 
 }  // namespace
@@ -294,6 +309,19 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
       DeviceGuard guard(device);
       if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes) == hipSuccess) {
         g->workspace_bytes = bytes;
+        // CCGLIB_AMD_INT1_OVERLAP=0 keeps everything on the caller's stream
+        const char *overlap = std::getenv("CCGLIB_AMD_INT1_OVERLAP");
+        if (!(overlap && std::strcmp(overlap, "0") == 0)) {
+          hipError_t e = hipStreamCreateWithFlags(&g->aux.stream, hipStreamNonBlocking);
+          if (e == hipSuccess) e = hipEventCreateWithFlags(&g->aux.fork, hipEventDisableTiming);
+          for (int i = 0; i < GemmAux::kMaxJoins && e == hipSuccess; ++i) {
+            e = hipEventCreateWithFlags(&g->aux.join[i], hipEventDisableTiming);
+          }
+          if (e != hipSuccess) {   // not an error: the GEMM then runs on one stream
+            release_aux(&g->aux);
+            (void)hipGetLastError();
+          }
+        }
       } else {
         g->workspace = nullptr;
         (void)hipGetLastError();
@@ -371,9 +399,11 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
 }
 
 int ccglib_gemm_destroy(ccglib_gemm_t g) {
-  if (g && g->workspace) {
+  if (g && (g->workspace || g->aux.stream)) {
     DeviceGuard guard(g->device);
-    (void)hipFree(g->workspace);   // waits for the kernels that still use it
+    if (g->aux.stream) (void)hipStreamSynchronize(g->aux.stream);
+    release_aux(&g->aux);
+    if (g->workspace) (void)hipFree(g->workspace);   // waits for the kernels that still use it
   }
   delete g;
   return CCGLIB_OK;

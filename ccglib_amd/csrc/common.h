@@ -56,6 +56,15 @@ inline int bits_of(int type) {
 // K values (samples) held by one 64-byte tile row.
 inline int k_per_tile(int type_in) { return kTileRowBytes * 8 / bits_of(type_in); }
 
+// A second stream with the events to fork from and join into the caller's
+// stream: work queued there may run beside the kernels on the caller's stream.
+struct GemmAux {
+  static constexpr int kMaxJoins = 8;
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr;
+  hipEvent_t join[kMaxJoins] = {};
+};
+
 // Problem description for one GEMM launch, in kernel terms. The kernel
 // computes D[y][x] = sum_k X[x][k] * Y[y][k] with x the contiguous output
 // axis: for a row-major C, X is the caller's B (N rows) and Y the caller's A
@@ -80,6 +89,9 @@ struct GemmParams {
   // 1-bit GEMM only: device memory for the operands expanded to fp4 (may be null)
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // 1-bit GEMM only: where the expansion of later batches may run while earlier
+  // batches are multiplied (may be null: everything on the one stream)
+  const GemmAux *aux = nullptr;
 };
 
 // Bytes of workspace with which the 1-bit GEMM of this size runs in one pass.

@@ -17,6 +17,8 @@
 // row is reused 8 times. Operand tiles have the same
 // 128-row x 64-byte geometry as the floating-point kernels and go through
 // the same global -> registers -> LDS double buffer.
+#include <algorithm>
+
 #include "gemm_device.h"
 
 namespace ccglib_amd {
@@ -329,39 +331,49 @@ __global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *
 // Largest K for which every partial sum (at most 2 K in magnitude) is exact in fp32.
 constexpr unsigned kMaxMfmaK = 1u << 22;
 
-hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *done) {
-  *done = false;
-  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
-  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
-  const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
-  const unsigned k_words = (unsigned)ceil_div(p.k, 32);
+// Batches per group when the expansion of one group of batches is to overlap
+// the multiplication of the previous one (the expansion is bound by memory
+// bandwidth, the multiplication by the matrix cores): the fewest batches that
+// give every compute unit a C tile, at most GemmAux::kMaxJoins groups; the
+// whole batch when that leaves fewer than two groups or there is no second
+// stream.
+size_t overlap_group(const GemmParams &p) {
+  if (!p.aux || !p.aux->stream) return p.batch;
+  const size_t tiles_per_batch = ceil_div(p.nx, 256) * ceil_div(p.ny, 128);
+  size_t group = ceil_div(256, tiles_per_batch);
+  group = std::max(group, ceil_div(p.batch, GemmAux::kMaxJoins));
+  return 2 * group <= p.batch ? group : p.batch;
+}
+
+// Expands (expand(b0, nb, ws_x, ws_y, stream)) and multiplies the batches in
+// groups of `group`; the workspace holds the groups one after the other when
+// `ws_advances`, else every group uses its start. With a second stream (only
+// when the workspace advances, so that no group overwrites what another still
+// needs) all expansions are queued there and each multiplication waits for its
+// own group's.
+template <typename Expand>
+hipError_t run_groups(const GemmParams &p, hipStream_t stream, size_t group, bool ws_advances,
+                      unsigned k4_tiles, Expand &&expand) {
   const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
   const size_t y_bytes = (size_t)p.y_tiles * k4_tiles * kTileBytes;
-  const size_t group = p.workspace_bytes / (x_bytes + y_bytes);
-  if (group == 0) return hipSuccess;
-  const bool tiled = (p.variant == kOpt);
-  if (!tiled && (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0)) return hipSuccess;
-  if (tiled && (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0)) return hipSuccess;
-  const size_t x_src = tiled ? (size_t)p.x_tiles * k1_tiles * kTileBytes : (size_t)2 * p.nx * k_words * 4;
-  const size_t y_src = tiled ? (size_t)p.y_tiles * k1_tiles * kTileBytes : (size_t)2 * p.ny * k_words * 4;
-  char *ws_x = static_cast<char *>(p.workspace);
-  for (size_t b0 = 0; b0 < p.batch; b0 += group) {
+  const bool overlap = ws_advances && p.aux && p.aux->stream && group < p.batch &&
+                       ceil_div(p.batch, group) <= (size_t)GemmAux::kMaxJoins;
+  hipStream_t expand_stream = overlap ? p.aux->stream : stream;
+  if (overlap) {
+    // the operands may still be being written on the caller's stream
+    if (hipError_t e = hipEventRecord(p.aux->fork, stream)) return e;
+    if (hipError_t e = hipStreamWaitEvent(p.aux->stream, p.aux->fork, 0)) return e;
+  }
+  char *ws = static_cast<char *>(p.workspace);
+  int gi = 0;
+  for (size_t b0 = 0; b0 < p.batch; b0 += group, ++gi) {
     const size_t nb = (p.batch - b0 < group) ? p.batch - b0 : group;
-    char *ws_y = ws_x + nb * x_bytes;
-    for (int which = 0; which < 2; ++which) {
-      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
-      const char *src = static_cast<const char *>(which ? p.y : p.x) + b0 * (which ? y_src : x_src);
-      char *dst = which ? ws_y : ws_x;
-      const size_t blocks = nb * row_tiles * k1_tiles;
-      if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-      const dim3 grid((unsigned)blocks, 4);
-      if (tiled) {
-        hipLaunchKernelGGL(expand_int1_to_fp4<true>, grid, dim3(256), 0, stream, src, dst, rows,
-                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
-      } else {
-        hipLaunchKernelGGL(expand_int1_to_fp4<false>, grid, dim3(256), 0, stream, src, dst, rows,
-                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
-      }
+    char *ws_x = ws, *ws_y = ws + nb * x_bytes;
+    if (ws_advances) ws += nb * (x_bytes + y_bytes);
+    if (hipError_t e = expand(b0, nb, ws_x, ws_y, expand_stream)) return e;
+    if (overlap) {
+      if (hipError_t e = hipEventRecord(p.aux->join[gi], p.aux->stream)) return e;
+      if (hipError_t e = hipStreamWaitEvent(stream, p.aux->join[gi], 0)) return e;
     }
     GemmParams q = p;
     q.x = ws_x;
@@ -374,8 +386,48 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
     q.input_interleaved = 0;
     if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
   }
-  *done = true;
   return hipGetLastError();
+}
+
+hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *done) {
+  *done = false;
+  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
+  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
+  const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
+  const unsigned k_words = (unsigned)ceil_div(p.k, 32);
+  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
+  const size_t y_bytes = (size_t)p.y_tiles * k4_tiles * kTileBytes;
+  const size_t fits = p.workspace_bytes / (x_bytes + y_bytes);
+  if (fits == 0) return hipSuccess;
+  const bool tiled = (p.variant == kOpt);
+  if (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0) return hipSuccess;
+  const size_t x_src = tiled ? (size_t)p.x_tiles * k1_tiles * kTileBytes : (size_t)2 * p.nx * k_words * 4;
+  const size_t y_src = tiled ? (size_t)p.y_tiles * k1_tiles * kTileBytes : (size_t)2 * p.ny * k_words * 4;
+  auto expand = [&](size_t b0, size_t nb, char *ws_x, char *ws_y, hipStream_t s) -> hipError_t {
+    for (int which = 0; which < 2; ++which) {
+      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+      const char *src = static_cast<const char *>(which ? p.y : p.x) + b0 * (which ? y_src : x_src);
+      char *dst = which ? ws_y : ws_x;
+      const size_t blocks = nb * row_tiles * k1_tiles;
+      if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+      const dim3 grid((unsigned)blocks, 4);
+      if (tiled) {
+        hipLaunchKernelGGL(expand_int1_to_fp4<true>, grid, dim3(256), 0, s, src, dst, rows,
+                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
+      } else {
+        hipLaunchKernelGGL(expand_int1_to_fp4<false>, grid, dim3(256), 0, s, src, dst, rows,
+                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
+      }
+    }
+    return hipSuccess;
+  };
+  // the whole problem in the workspace: groups chosen for overlap, laid out one
+  // after the other; a smaller workspace: as many batches at a time as fit
+  const bool whole = fits >= p.batch;
+  const size_t group = whole ? overlap_group(p) : fits;
+  if (hipError_t e = run_groups(p, stream, group, whole, k4_tiles, expand)) return e;
+  *done = true;
+  return hipSuccess;
 }
 
 }  // namespace
@@ -389,32 +441,25 @@ bool gemm_int1_can_take_bytes(const GemmParams &p) {
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
   if (!gemm_int1_can_take_bytes(p)) return hipErrorInvalidValue;
   const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
-  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
-  char *ws_x = static_cast<char *>(p.workspace);
-  char *ws_y = ws_x + p.batch * x_bytes;
-  for (int which = 0; which < 2; ++which) {
-    const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
-    const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
-    char *dst = which ? ws_y : ws_x;
-    const dim3 grid((unsigned)ceil_div(k4_tiles, 4), 2 * row_tiles, 2 * p.batch);
-    const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
-    if (vec) {
-      hipLaunchKernelGGL(expand_bytes_to_fp4<true>, grid, dim3(256), 0, stream, src, dst, rows,
-                         row_tiles, p.k, k4_tiles);
-    } else {
-      hipLaunchKernelGGL(expand_bytes_to_fp4<false>, grid, dim3(256), 0, stream, src, dst, rows,
-                         row_tiles, p.k, k4_tiles);
+  auto expand = [&](size_t b0, size_t nb, char *ws_x, char *ws_y, hipStream_t s) -> hipError_t {
+    for (int which = 0; which < 2; ++which) {
+      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+      const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x) +
+                                 b0 * 2 * (size_t)rows * p.k;
+      char *dst = which ? ws_y : ws_x;
+      const dim3 grid((unsigned)ceil_div(k4_tiles, 4), 2 * row_tiles, 2 * (unsigned)nb);
+      const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
+      if (vec) {
+        hipLaunchKernelGGL(expand_bytes_to_fp4<true>, grid, dim3(256), 0, s, src, dst, rows,
+                           row_tiles, p.k, k4_tiles);
+      } else {
+        hipLaunchKernelGGL(expand_bytes_to_fp4<false>, grid, dim3(256), 0, s, src, dst, rows,
+                           row_tiles, p.k, k4_tiles);
+      }
     }
-  }
-  GemmParams q = p;
-  q.x = ws_x;
-  q.y = ws_y;
-  q.k_tiles = k4_tiles;
-  q.type_in = kFp4Sign;
-  q.variant = kOpt;
-  q.input_interleaved = 0;
-  if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
-  return hipGetLastError();
+    return hipSuccess;
+  };
+  return run_groups(p, stream, overlap_group(p), true, k4_tiles, expand);
 }
 
 size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k) {

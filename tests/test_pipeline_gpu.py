@@ -1,5 +1,7 @@
 """GPU parity tests of the pipeline wrapper (pack -> transpose -> GEMM) against the
 CPU oracle; cases follow the reference's test/pipeline/pipeline.cpp."""
+import functools
+
 import numpy as np
 import pytest
 import torch
@@ -132,6 +134,48 @@ def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
     once = orc.gemm(pa, pb, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, c_in)
     want = orc.gemm(pa, pb, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, once.reshape(-1))
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+
+
+@functools.lru_cache(maxsize=1)
+def _grouped_int1_case(B, M, N, K):
+    """Two sets of random 1-bit operands (one byte per sample) and the oracle's C for each."""
+    rng = np.random.default_rng(77)
+    bits = [[rng.integers(0, 2, B * 2 * rows * K, dtype=np.uint8) for rows in (M, N)] for _ in range(2)]
+    wants = [orc.gemm(orc.pack_bits(a), orc.pack_bits(b), M, N, K, orc.INT1, orc.INT32) for a, b in bits]
+    return bits, wants
+
+
+@pytest.mark.parametrize("overlap", [True, False])
+@pytest.mark.parametrize("what", ["pipeline", "gemm_opt", "gemm_basic"])
+def test_int1_expansion_in_groups(what, overlap, monkeypatch):
+    """Enough batches and C tiles (16 x 32 tiles of 256 x 128) for the 1-bit GEMM to expand and
+    multiply in two groups of 8 batches, the expansion on a second stream (or, with
+    CCGLIB_AMD_INT1_OVERLAP=0, everything on the caller's stream). Two Runs in a row with
+    different input: the second call's expansion must not overtake the first call's GEMMs."""
+    if not overlap:
+        monkeypatch.setenv("CCGLIB_AMD_INT1_OVERLAP", "0")
+    B, M, N, K = 16, 1024, 1024, 256
+    bits, wants = _grouped_int1_case(B, M, N, K)
+    d_c = [to_device(np.zeros(B * 2 * M * N, dtype=np.int32)) for _ in range(2)]
+    if what == "pipeline":
+        obj = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                          cc.Variant.opt)
+        d_in = [[to_device(x) for x in pair] for pair in bits]
+    else:
+        variant = cc.Variant.opt if what == "gemm_opt" else cc.Variant.basic
+        obj = cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.int1, VT.int32), variant)
+        packed = [[orc.pack_bits(x) for x in pair] for pair in bits]
+        if what == "gemm_opt":
+            from gpu_util import transpose_operand
+            d_in = [[transpose_operand(x, B, rows, K, VT.int1) for x, rows in zip(pair, (M, N))]
+                    for pair in packed]
+        else:
+            d_in = [[to_device(x) for x in pair] for pair in packed]
+    for i in range(2):
+        obj.Run(d_in[i][0].data_ptr(), d_in[i][1].data_ptr(), d_c[i].data_ptr())
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert np.array_equal(to_host(d_c[i], np.int32).reshape(wants[i].shape), wants[i])
 
 
 def pack_rows(bits, B, rows, K):
