@@ -814,6 +814,49 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
   }
 }
 
+// The same for planar fp16 / bf16 C: a tile row of 16 x 64 values is 16 rows of
+// 128 bytes (stride 144 in the patch: conflict-free 8-byte writes down a column,
+// 16-byte aligned reads along a row); every store instruction writes eight whole
+// 128-byte row segments instead of sixteen 32-byte pieces.
+template <int TOUT, int TX, int TY>
+__device__ __forceinline__ void store_wave_tile_staged_narrow(const KernelArgs &args, unsigned b,
+                                                              unsigned x_wave, unsigned y_wave,
+                                                              int lane, char *patch,
+                                                              float4_t (&acc_re)[TY][TX],
+                                                              float4_t (&acc_im)[TY][TX]) {
+  static_assert(TX == 4, "patch rows hold 64 columns");
+  using Tout = typename OutType<TOUT>::type;
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha;
+  const float ar = args.alpha_re, ai = args.alpha_im;
+  Tout *cbase = reinterpret_cast<Tout *>(args.c) + (size_t)b * 2 * nx * ny;
+  char *wr = patch + (lane & 15) * 144 + (lane >> 4) * 8;        // [y = lane%16][x = (lane/16)*4 ..]
+  const char *rd = patch + (lane >> 3) * 144 + (lane & 7) * 16;  // [row lane/8][x = (lane%8)*8 ..]
+  Tout *out = cbase + (size_t)(y_wave + (lane >> 3)) * nx + x_wave + (lane & 7) * 8;
+#pragma unroll
+  for (int plane = 0; plane < 2; ++plane) {
+#pragma unroll
+    for (int j = 0; j < TY; ++j) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i) {
+        Tout v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float re = acc_re[j][i][e], im = acc_im[j][i][e];
+          v[e] = (Tout)(plane == 0 ? (have_alpha ? ar * re - ai * im : re)
+                                   : (have_alpha ? ai * re + ar * im : im));
+        }
+        *reinterpret_cast<ushort4_t *>(wr + i * 32) = __builtin_bit_cast(ushort4_t, v);
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int4_t v = *reinterpret_cast<const int4_t *>(rd + r * 8 * 144);
+        *reinterpret_cast<int4_t *>(out + (size_t)plane * nx * ny + (size_t)(j * 16 + r * 8) * nx) = v;
+      }
+    }
+  }
+}
+
 // The same for interleaved fp32 C: 16 rows of 32 (re, im) pairs at a time (half
 // the width of the wave tile, again 256 bytes per row) go through the patch.
 template <int TX, int TY>
@@ -1337,6 +1380,20 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           } else {
             store_wave_tile_staged<TX, TY>(args, tc.b, x_wave, y_wave, lane, patch, acc_re, acc_im);
           }
+          staged = true;
+        }
+      }
+    }
+    if constexpr (MS == 16 && (TOUT == kFloat16 || TOUT == kBfloat16) && TX == 4 &&
+                  NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
+      if (staged_ok && !args.c_interleaved && args.nx % 8 == 0) {
+        unsigned free_slot = slot + LEAD * KPI;
+        free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
+        asm volatile("s_barrier" ::: "memory");
+        if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
+          store_wave_tile_staged_narrow<TOUT, TX, TY>(
+              args, tc.b, x_wave, y_wave, lane,
+              lds + free_slot * SLOT_BYTES + wave * kStagePatchBytes, acc_re, acc_im);
           staged = true;
         }
       }

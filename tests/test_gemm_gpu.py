@@ -180,6 +180,17 @@ def test_interleaved_c_alpha_only(tin, c_order):
     float_case(2, 256, 512, 64, tin, VT.float32, cc.Variant.opt, INTERLEAVED, c_order, seed=22)
 
 
+@pytest.mark.parametrize("c_order", [ROW, COL])
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float16), (VT.bfloat16, VT.bfloat16),
+                                      (VT.float32, VT.float16), (VT.float32, VT.bfloat16)])
+def test_narrow_planar_c_alpha_only(tin, tout, c_order):
+    # 16-bit planar C, beta = 0, rows of whole 16-byte vectors: wave tiles inside C take the
+    # LDS-staged stores, the ragged edges (M = 300, N = 328) the direct ones
+    float_case(3, 300, 328, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=0.75 - 0.5j, seed=23)
+    float_case(2, 256, 512, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=24)
+    float_case(2, 256, 516, 64, tin, tout, cc.Variant.basic, PLANAR, c_order, seed=25)   # N % 8 != 0: direct
+
+
 def test_fp32_alpha_beta_and_many_tiles():
     float_case(3, 256, 320, 96, VT.float32, VT.float32, cc.Variant.opt, INTERLEAVED, COL,
                alpha=0.75 - 0.5j, beta=0.5 - 0.25j)
