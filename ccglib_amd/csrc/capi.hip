@@ -670,15 +670,14 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   // GEMM as it is (the kernel de-interleaves in its arithmetic), which saves the
   // two transposes and their intermediate buffers for either variant.
   const size_t in_bits = (size_t)bits_of(input_type);
-  // Reading rows in place costs the GEMM 6-9 % (16-bit) or, with the smaller
-  // block of the 8-bit kernel, almost 50 % against reading tiles; the transposes
-  // cost two bandwidth-bound passes over A and B. The first is the smaller price
-  // while M N / (M + N) stays below about 2800 (16-bit) or 330 (8-bit input),
-  // from the measured rates of the kernels involved.
+  // Reading rows in place costs the GEMM 6-9 % against reading tiles; the
+  // transposes cost two bandwidth-bound passes over A and B. The first is the
+  // smaller price while M N / (M + N) stays below about 2800 (16-bit) or 3000
+  // (8-bit input), from the measured rates of the kernels involved.
   const double mn_over_sum = (M + N) ? (double)M * (double)N / (double)(M + N) : 0.0;
   const bool fused = !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&
-                     (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2800.0 : 330.0));
+                     (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2800.0 : 3000.0));
   // The reference transposes for the opt variant only (:53) and hands interleaved
   // input of the basic variant to a kernel that reads it as planar. Here such
   // input is always de-interleaved: in the GEMM's loader (fused) or, where that

@@ -590,6 +590,86 @@ __device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, c
 #undef CCGLIB_PIN
 }
 
+// Interleaved 8-bit operands on the 32-row MFMA: a 2 x 2 wave tile of 32 x 32
+// tiles; the slot holds 128 bytes (64 (re, im) pairs) of every row, walked in two
+// halves of 64 bytes, one MFMA step each. off[h][u] are the lane's two 16-byte
+// chunks of its row in half h. As for 16-bit input the raw X fragment is used
+// as it is and both Y variants come from the raw Y fragment: a sign flip of the
+// odd bytes and a swap inside each byte pair. LDS reads are placed by hand, a
+// fragment being fetched about four MFMAs (of 32 cycles) ahead of its use.
+template <int DT, int BX, int BY, typename Mid>
+__device__ __forceinline__ void mma_step32_interleaved(const char *slot, const int (&x_off)[2][2],
+                                                       const int (&y_off)[2][2],
+                                                       float16_t_ (&acc_re)[2][2],
+                                                       float16_t_ (&acc_im)[2][2], Mid &&mid) {
+  static_assert(DtypeTraits<DT>::kElemBytes == 1, "8-bit input");
+  auto rd = [&](const int (&off)[2], int extra) {
+    Fragment32 f;
+    f.v[0] = *reinterpret_cast<const int4_t *>(slot + off[0] + extra);
+    f.v[1] = *reinterpret_cast<const int4_t *>(slot + off[1] + extra);
+    return f;
+  };
+  auto flip = [](const Fragment32 &raw) {      // (yr, -yi, ...)
+    Fragment32 f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) f.v[u][w] = (int)((unsigned)raw.v[u][w] ^ 0x80008000u);
+    }
+    return f;
+  };
+  auto swap = [](const Fragment32 &raw) {      // (yi, yr, ...)
+    Fragment32 f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned v = (unsigned)raw.v[u][w];
+        f.v[u][w] = (int)__builtin_amdgcn_perm(v, v, 0x02030001u);
+      }
+    }
+    return f;
+  };
+  constexpr int ROW32 = 32 * 128;
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+  Fragment32 x0, x1, raw0, raw1, ya, yb;
+  raw0 = rd(y_off[0], 0);
+  x0 = rd(x_off[0], 0);
+  x1 = rd(x_off[0], ROW32);
+  CCGLIB_PIN;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    ya = flip(raw0);
+    yb = swap(raw0);
+    CCGLIB_PIN;
+    acc_re[0][0] = mfma32<DT>(x0, ya, acc_re[0][0]);
+    raw1 = rd(y_off[h], ROW32);
+    CCGLIB_PIN;
+    acc_im[0][0] = mfma32<DT>(x0, yb, acc_im[0][0]);
+    CCGLIB_PIN;
+    if (h == 0) {
+      mid();
+      CCGLIB_PIN;
+    }
+    acc_re[0][1] = mfma32<DT>(x1, ya, acc_re[0][1]);
+    if (h == 0) raw0 = rd(y_off[1], 0);
+    CCGLIB_PIN;
+    acc_im[0][1] = mfma32<DT>(x1, yb, acc_im[0][1]);
+    ya = flip(raw1);
+    yb = swap(raw1);
+    CCGLIB_PIN;
+    acc_re[1][0] = mfma32<DT>(x0, ya, acc_re[1][0]);
+    acc_im[1][0] = mfma32<DT>(x0, yb, acc_im[1][0]);
+    if (h == 0) x0 = rd(x_off[1], 0);
+    CCGLIB_PIN;
+    acc_re[1][1] = mfma32<DT>(x1, ya, acc_re[1][1]);
+    acc_im[1][1] = mfma32<DT>(x1, yb, acc_im[1][1]);
+    if (h == 0) x1 = rd(x_off[1], ROW32);
+    CCGLIB_PIN;
+  }
+#undef CCGLIB_PIN
+}
+
 // Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
 // store, piece by piece (four consecutive elements of the contiguous C axis).
 template <int TOUT, int TX, int TY, int MS = 16, typename Acc>
@@ -1130,8 +1210,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
   constexpr int TX = WX / MS, TY = WY / MS;          // MFMA tiles of a wave
   constexpr int KPM = MS == 32 ? 1 : DtypeTraits<DT>::kTilesPerMfma;
-  static_assert(MS == 16 || (MS == 32 && LOADER != kLoadInterleavedVec),
-                "the 32-row MFMAs are used for planar operands");
+  static_assert(MS == 16 || LOADER != kLoadInterleavedVec || DtypeTraits<DT>::kElemBytes == 1,
+                "interleaved operands on the 32-row MFMAs: 8-bit input only");
   // interleaved operands: one plane of (re, im) rows
   // (their slots hold 128 bytes of every row, fetched as whole cache lines)
   constexpr bool IL = (LOADER == kLoadInterleavedVec);
@@ -1176,7 +1256,12 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int r = lane / CPR;                                   // row inside the row block
   // chunk that belongs at lane*16: the XOR pattern that makes the fragment
   // reads of the MFMA shape in use free of bank conflicts (measured)
+  // (interleaved rows on the 32-row MFMAs: XOR with (row >> 1) & 7, which also
+  // depends on the parity of the 8-row row block, see c_of below)
   const int c = (lane % CPR) ^ (IL ? r & 7 : MS == 32 ? (r >> 2) & 3 : (r >> 1) & 3);
+  auto c_of = [&](int rb) {   // chunk this lane fetches for row block rb of an operand
+    return (IL && MS == 32) ? ((lane % CPR) ^ (((rb & 1) << 2) | ((r >> 1) & 3))) : c;
+  };
   {
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
@@ -1215,7 +1300,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           const unsigned total_rows = is_x ? args.nx : args.ny;
           unsigned row = row0 + r;
           row = row < total_rows ? row : total_rows - 1;   // likewise
-          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_bytes + c * 16;
+          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_bytes + c_of(rb) * 16;
         }
       }
     }
@@ -1235,9 +1320,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
-      const bool inside = (load_kt * RB + c * 16 + 16 <= row_bytes);
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
+        const int q = i * NW + wave;
+        const int rb = (q < X_ROW_BLOCKS ? q : q - X_ROW_BLOCKS) % ((q < X_ROW_BLOCKS ? BX : BY) / RPB);
+        const bool inside = (load_kt * RB + c_of(rb) * 16 + 16 <= row_bytes);
         const char *p = inside ? lane_src[i] + (size_t)load_kt * RB
                                : g_zero_tile + lane * 16;
         load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
@@ -1275,6 +1362,19 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int xil_off[2] = {(wx * WX) * 128 + il_off[0], (wx * WX) * 128 + il_off[1]};
   const int yil_off[2] = {X_BYTES + (wy * WY) * 128 + il_off[0],
                           X_BYTES + (wy * WY) * 128 + il_off[1]};
+  // interleaved rows on the 32-row MFMAs: row lane % 32, half h of the 128 bytes, chunks
+  // 4 h + 2 (lane / 32) and the next one
+  int xil32_off[2][2], yil32_off[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int row = lane & 31, chunk = 4 * h + 2 * (lane >> 5) + u;
+      const int off = row * 128 + ((chunk ^ ((row >> 1) & 7)) * 16);
+      xil32_off[h][u] = (wx * WX) * 128 + off;
+      yil32_off[h][u] = X_BYTES + (wy * WY) * 128 + off;
+    }
+  }
   // wide stores through LDS: no beta term, vector-aligned rows (interleaved C
   // only with the 16-row layout)
   const bool staged_ok = (MS == 16 || !args.c_interleaved) && !args.have_beta &&
@@ -1332,7 +1432,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           for (int u = 0; u < KPI; ++u) issue_next(refill + u);
         }
       };
-      if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
+      if constexpr (IL && MS == 32) {
+        static_assert(TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
+        mma_step32_interleaved<DT, BX, BY>(lds + slot * SLOT_BYTES, xil32_off, yil32_off, acc_re,
+                                           acc_im, refill_slots);
+      } else if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
         mma_step_interleaved_ordered<DT, BX, BY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
                                                  acc_im, refill_slots);
       } else if constexpr (IL) {
@@ -1514,7 +1618,7 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     } else if constexpr (KPM == 1) {
       return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec>(p, stream);
     } else {
-      return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec>(p, stream);
+      return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>(p, stream);
     }
   }
   if (p.variant == kOpt || planar_direct) {

@@ -51,6 +51,7 @@ static const std::vector<Config> kConfigs = {
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
     {"fp8 interleaved 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec, 16>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
+    {"fp8 interleaved 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
 };
 
 static double peak_of(int type) {

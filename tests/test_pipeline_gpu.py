@@ -290,10 +290,10 @@ def test_pipeline_interleaved_input(tin, tout, K, variant):
 
 @pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
 def test_pipeline_interleaved_input_large_c(tin):
-    # With M N / (M + N) above about 2800 (330 for 8-bit input) the opt pipeline transposes
+    # With M N / (M + N) above about 2800 (3000 for 8-bit input) the opt pipeline transposes
     # interleaved input into tiles instead of reading the rows in place (the GEMM then runs
     # enough faster to pay for the two transposes); same numbers either way.
-    B, M, N, K = 1, 6144, 6144, 64
+    B, M, N, K = 1, 6144, 6144, 64      # M N / (M + N) = 3072
     rng = np.random.default_rng(31)
     qa = quantize(rng.uniform(-1, 1, B * 2 * M * K), tin)
     qb = quantize(rng.uniform(-1, 1, B * 2 * N * K), tin)
