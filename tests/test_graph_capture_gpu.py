@@ -1,0 +1,116 @@
+"""Run() only enqueues work on the stream the object was created with and allocates
+nothing, so it can be captured into a HIP graph: the graph is replayed several times
+on changed input, with eager work and synchronisations in between, and every replay
+is compared with the eager result."""
+import numpy as np
+import pytest
+import torch
+
+import ccglib_amd as cc
+from gpu_util import quantize, to_device, transpose_operand
+
+pytestmark = pytest.mark.gpu
+VT = cc.ValueType
+PLANAR, INTERLEAVED = cc.ComplexAxisLocation.complex_planar, cc.ComplexAxisLocation.complex_interleaved
+ROW, COL = cc.MemOrder.row_major, cc.MemOrder.col_major
+
+
+def _capture_and_replay(make_object, inputs, fill_inputs, out_shape, out_dtype, rounds=3):
+    """make_object(stream) -> object with Run(a, b, c); inputs: list of device tensors the
+    graph reads; fill_inputs(round) writes new contents into them."""
+    side = torch.cuda.Stream()
+    obj = make_object(side.cuda_stream)
+    d_c = torch.zeros(out_shape, dtype=out_dtype, device="cuda")
+    fill_inputs(0)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):           # warm-up outside the capture
+        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+    for r in range(1, rounds + 1):
+        fill_inputs(r)
+        torch.cuda.synchronize()
+        d_c.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = d_c.clone()
+        d_c.zero_()
+        with torch.cuda.stream(side):
+            obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(got, d_c), "replay %d differs from the eager run" % r
+        assert bool(d_c.ne(0).any())
+
+
+def test_graph_gemm_fp16_opt():
+    B, M, N, K = 4, 256, 384, 128
+    a = transpose_operand(quantize(np.zeros(B * 2 * M * K), VT.float16), B, M, K, VT.float16)
+    b = transpose_operand(quantize(np.zeros(B * 2 * N * K), VT.float16), B, N, K, VT.float16)
+
+    def fill(r):
+        g = torch.Generator(device="cuda").manual_seed(100 + r)
+        for t in (a, b):   # any bit pattern of small fp16 numbers, tile padding included
+            t.copy_(torch.randint(0, 64, t.shape, generator=g, device="cuda", dtype=torch.uint8))
+
+    _capture_and_replay(lambda s: cc.GEMM(B, M, N, K, 0, s, cc.Precision(VT.float16, VT.float32),
+                                          cc.Variant.opt),
+                        [a, b], fill, (B * 2 * M * N,), torch.float32)
+
+
+def test_graph_pipeline_fp16_interleaved():
+    B, M, N, K = 3, 256, 512, 96
+    a = torch.zeros(B * M * K * 2, dtype=torch.float16, device="cuda")
+    b = torch.zeros(B * N * K * 2, dtype=torch.float16, device="cuda")
+
+    def fill(r):
+        g = torch.Generator(device="cuda").manual_seed(200 + r)
+        for t in (a, b):
+            t.copy_(torch.randn(t.shape, generator=g, device="cuda").to(torch.float16))
+
+    _capture_and_replay(lambda s: cc.Pipeline(B, M, N, K, 0, s, INTERLEAVED, PLANAR, ROW, COL, ROW,
+                                              VT.float16, VT.float32, cc.Variant.opt),
+                        [a, b], fill, (B * 2 * M * N,), torch.float32)
+
+
+@pytest.mark.parametrize("what", ["pipeline", "packing_transpose_gemm"])
+def test_graph_int1(what):
+    # 16 batches of 32 C tiles: the 1-bit GEMM expands and multiplies in two groups, the
+    # expansions on the object's second stream, forked from and joined into the captured one
+    B, M, N, K = 16, 1024, 1024, 256
+    a = torch.zeros(B * 2 * M * K, dtype=torch.uint8, device="cuda")
+    b = torch.zeros(B * 2 * N * K, dtype=torch.uint8, device="cuda")
+
+    def fill(r):
+        g = torch.Generator(device="cuda").manual_seed(300 + r)
+        for t in (a, b):
+            t.copy_(torch.randint(0, 2, t.shape, generator=g, device="cuda", dtype=torch.uint8))
+
+    if what == "pipeline":
+        make = lambda s: cc.Pipeline(B, M, N, K, 0, s, PLANAR, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                                     cc.Variant.opt)
+    else:
+        class Steps:
+            """Packing -> Transpose -> GEMM as separate objects on one stream."""
+            def __init__(self, s):
+                prec = cc.Precision(VT.int1, VT.int32)
+                mb, nb, kc = cc.GEMM.GetDimensions(prec)
+                self.pk = [cc.Packing(B * 2 * rows * K, cc.Direction.forward, 0, s) for rows in (M, N)]
+                self.tr = [cc.Transpose(B, rows, K, mb, kc, 1, 0, s) for rows in (M, N)]
+                self.packed = [torch.zeros(B * 2 * rows * K // 32, dtype=torch.int32, device="cuda")
+                               for rows in (M, N)]
+                # the tiled layout holds whole tiles: rows padded to mb / nb, K to kc (512 samples)
+                kp = cc.ceildiv(K, kc) * kc
+                self.tiled = [torch.zeros(B * 2 * (cc.ceildiv(rows, t) * t) * kp // 32, dtype=torch.int32,
+                                          device="cuda") for rows, t in ((M, mb), (N, nb))]
+                self.gemm = cc.GEMM(B, M, N, K, 0, s, prec, cc.Variant.opt)
+
+            def Run(self, pa, pb, pc):
+                for i, src in enumerate((pa, pb)):
+                    self.pk[i].Run(src, self.packed[i].data_ptr())
+                    self.tr[i].Run(self.packed[i].data_ptr(), self.tiled[i].data_ptr())
+                self.gemm.Run(self.tiled[0].data_ptr(), self.tiled[1].data_ptr(), pc)
+        make = Steps
+
+    _capture_and_replay(make, [a, b], fill, (B * 2 * M * N,), torch.int32)
