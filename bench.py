@@ -1,6 +1,6 @@
 """Benchmark of the hot path on one MI355X.
 
-Default workload (the one the headline metric is quoted on, BASELINE.json configs[1]):
+Default workload (the configuration the reference's headline metric is quoted on):
 a step is one pass over one batch of synthetic input of the beamformer-shaped
 problem: interleaved fp16 A [64][512][576][2] (unit-magnitude random phases) and
 B [64][4096][576][2] (complex Gaussian, sigma 1) are brought into the tiled layout
@@ -11,8 +11,8 @@ Prints one JSON line. `value` is 8*B*M*N*K / (time per step): the whole step, da
 preparation kernels (transpose, packing) included. The `roofline` object is about the
 GEMM kernel alone, timed with events on the launch stream inside the timed region.
 
-Other workloads (`--workload`): the remaining BASELINE.json configurations, for the
-per-kernel tables in DESIGN.md; the driver's default run does not use them.
+Other workloads (`--workload`): the reference's other benchmark configurations, for
+per-kernel measurements; a run without flags does not use them.
 """
 import argparse
 import json

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes. The CPU oracle cannot finish these
+"""The reference's benchmark configurations at their full sizes. The CPU oracle cannot finish these
 in reasonable time, so they are checked through properties that do not depend on size:
 one batch against an independent float64 (or exact +-1) product computed by torch on
 the GPU, CPU-oracle spot blocks with the full K, bit-exact transposes against torch's
