@@ -290,41 +290,48 @@ __global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *
                                                            char *__restrict__ dst, unsigned rows,
                                                            unsigned row_tiles, unsigned k,
                                                            unsigned k4_tiles) {
-  // blockIdx: x = group of four K tiles of 128 samples, y = block of 64 rows, z = (batch, plane);
-  // a thread takes quarter c of each of the four K tiles (eight 16-byte loads in flight)
-  const unsigned c = threadIdx.x & 3, row_in_tile = (blockIdx.y & 1) * 64 + (threadIdx.x >> 2);
+  // blockIdx: x = group of four K tiles of 128 samples (512 bytes of a row), y = block of 64
+  // rows, z = (batch, plane). A wave takes 16 rows, four at a time: lane = (row of the four,
+  // 32-sample piece of the 512), so that a load instruction reads four runs of 512
+  // contiguous bytes; a thread has eight 16-byte loads in flight (four rows, two each) and
+  // writes four 16-byte pieces (a store instruction writes 256 contiguous bytes in each of
+  // four K tiles).
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned piece = lane & 15, s = piece >> 2, c = piece & 3;
   const unsigned rt = blockIdx.y >> 1;
   const size_t b = blockIdx.z >> 1;
   const unsigned plane = blockIdx.z & 1;
-  const unsigned r = rt * kTileRows + row_in_tile;
-  const unsigned char *row_ptr = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
-  unsigned bits[4], n[4];
+  const unsigned k4 = 4 * blockIdx.x + s;
+  const unsigned k0 = k4 * 128 + c * 32;
+  unsigned row_in_tile[4], n[4];
+  const unsigned char *row_ptr[4];
   uint4_t v[4][2];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const unsigned k0 = (4 * blockIdx.x + s) * 128 + c * 32;
-    n[s] = (r < rows && k0 < k) ? (k - k0 < 32 ? k - k0 : 32) : 0;
-    if (VEC && n[s] == 32) {
-      v[s][0] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr + k0));
-      v[s][1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr + k0) + 1);
+  for (int q = 0; q < 4; ++q) {
+    row_in_tile[q] = (blockIdx.y & 1) * 64 + wave * 16 + q * 4 + (lane >> 4);
+    const unsigned r = rt * kTileRows + row_in_tile[q];
+    row_ptr[q] = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
+    n[q] = (r < rows && k0 < k) ? (k - k0 < 32 ? k - k0 : 32) : 0;
+    if (VEC && n[q] == 32) {
+      v[q][0] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0));
+      v[q][1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0) + 1);
     }
   }
+  if (k4 >= k4_tiles) return;
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const unsigned k4 = 4 * blockIdx.x + s;
-    if (k4 >= k4_tiles) break;
-    const unsigned k0 = k4 * 128 + c * 32;
-    if (VEC && n[s] == 32) {
-      bits[s] = nonzero_bits_of16(v[s][0]) | (nonzero_bits_of16(v[s][1]) << 16);
+  for (int q = 0; q < 4; ++q) {
+    unsigned bits;
+    if (VEC && n[q] == 32) {
+      bits = nonzero_bits_of16(v[q][0]) | (nonzero_bits_of16(v[q][1]) << 16);
     } else {
-      bits[s] = 0;
-      for (unsigned i = 0; i < n[s]; ++i) bits[s] |= (row_ptr[k0 + i] != 0 ? 1u : 0u) << i;
+      bits = 0;
+      for (unsigned i = 0; i < n[q]; ++i) bits |= (row_ptr[q][k0 + i] != 0 ? 1u : 0u) << i;
     }
-    const unsigned valid = n[s] == 32 ? 0xffffffffu : ((1u << n[s]) - 1u);
-    const uint4_t o = nibbles_of(bits[s], valid);
+    const unsigned valid = n[q] == 32 ? 0xffffffffu : ((1u << n[q]) - 1u);
+    const uint4_t o = nibbles_of(bits, valid);
     __builtin_nontemporal_store(
         o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
-                                       plane * kTilePlaneBytes + row_in_tile * kTileRowBytes + 16 * c));
+                                       plane * kTilePlaneBytes + row_in_tile[q] * kTileRowBytes + 16 * c));
   }
 }
 
