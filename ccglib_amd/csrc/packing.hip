@@ -122,15 +122,32 @@ __global__ __launch_bounds__(256) void pack_scalar(const unsigned char *__restri
   out[w] = v;
 }
 
-// thread -> 16 output bytes from half a word.
+// thread -> four times 16 output bytes, each from half a word: four small loads
+// in flight per thread (with one, the kernel waits on the latency of its reads),
+// and every store instruction of a wave writes 1 KiB contiguous.
+constexpr int kUnpackPerThread = 4;
 __global__ __launch_bounds__(256) void unpack_vec(const unsigned *__restrict__ in,
                                                   uint4_t *__restrict__ out, size_t n16) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < n16; g += stride) {
-    const unsigned h = (in[g >> 1] >> ((g & 1) * 16)) & 0xffffu;
-    __builtin_nontemporal_store(uint4_t{bytes_of_nibble(h), bytes_of_nibble(h >> 4),
-                                        bytes_of_nibble(h >> 8), bytes_of_nibble(h >> 12)},
-                                out + g);
+  const size_t stride = (size_t)gridDim.x * 256 * kUnpackPerThread;
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kUnpackPerThread; base < n16;
+       base += stride) {
+    unsigned w[kUnpackPerThread];
+#pragma unroll
+    for (int k = 0; k < kUnpackPerThread; ++k) {
+      const size_t g = base + k * 64 + lane;
+      w[k] = g < n16 ? __builtin_nontemporal_load(in + (g >> 1)) : 0u;
+    }
+#pragma unroll
+    for (int k = 0; k < kUnpackPerThread; ++k) {
+      const size_t g = base + k * 64 + lane;
+      if (g < n16) {
+        const unsigned h = (w[k] >> ((g & 1) * 16)) & 0xffffu;
+        __builtin_nontemporal_store(uint4_t{bytes_of_nibble(h), bytes_of_nibble(h >> 4),
+                                            bytes_of_nibble(h >> 8), bytes_of_nibble(h >> 12)},
+                                    out + g);
+      }
+    }
   }
 }
 
@@ -190,7 +207,7 @@ hipError_t launch_unpack_bits(const unsigned *in, unsigned char *out, size_t n,
   size_t done = 0;
   if ((uintptr_t)out % 16 == 0 && n >= 16) {
     const size_t n16 = n / 16;
-    hipLaunchKernelGGL(unpack_vec, dim3(grid_for(n16, 1)), dim3(256), 0, stream, in,
+    hipLaunchKernelGGL(unpack_vec, dim3(grid_for(n16, kUnpackPerThread)), dim3(256), 0, stream, in,
                        reinterpret_cast<uint4_t *>(out), n16);
     done = n16 * 16;
   }
