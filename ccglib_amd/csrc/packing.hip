@@ -35,26 +35,29 @@ __device__ __forceinline__ unsigned bytes_of_nibble(unsigned b) {
 
 constexpr int kUnroll = 1;
 
-// Planar: thread -> 16 input bytes -> half an output word; lane pairs merge.
+// Planar: thread -> kPackPerThread times 16 input bytes, each half an output word;
+// lane pairs merge. A wave takes 64 * kPackPerThread consecutive groups, so every
+// load instruction reads 1 KiB contiguous and a thread has several in flight.
 // n16 = number of whole 16-byte groups that make whole words (2 per word).
+constexpr int kPackPerThread = 2;
 __global__ __launch_bounds__(256) void pack_planar_vec(const uint4_t *__restrict__ in,
                                                        unsigned *__restrict__ out, size_t n16) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-  // n16 is even and the stride is even, so a lane pair is in or out together
-  for (; g < n16; g += stride * kUnroll) {
-    uint4_t v[kUnroll];
+  const size_t stride = (size_t)gridDim.x * 256 * kPackPerThread;
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // n16 and every item index base + 64 k are even, so a lane pair is in or out together
+  for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kPackPerThread; base < n16; base += stride) {
+    uint4_t v[kPackPerThread];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const size_t gi = g + u * stride;
-      v[u] = gi < n16 ? __builtin_nontemporal_load(in + gi) : uint4_t{0, 0, 0, 0};
+    for (int k = 0; k < kPackPerThread; ++k) {
+      const size_t gi = base + k * 64 + lane;
+      v[k] = gi < n16 ? __builtin_nontemporal_load(in + gi) : uint4_t{0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const size_t gi = g + u * stride;
-      const unsigned mine = bits_of16(v[u]);
+    for (int k = 0; k < kPackPerThread; ++k) {
+      const size_t gi = base + k * 64 + lane;
+      const unsigned mine = bits_of16(v[k]);
       const unsigned next = __shfl_down(mine, 1);
-      if ((threadIdx.x & 1) == 0 && gi < n16) out[gi >> 1] = mine | (next << 16);
+      if ((lane & 1) == 0 && gi < n16) out[gi >> 1] = mine | (next << 16);
     }
   }
 }
@@ -182,7 +185,7 @@ hipError_t launch_pack_bits(const unsigned char *in, unsigned *out, size_t n, in
     vec_words = n / 32;
     if (vec_words) {
       const size_t n16 = vec_words * 2;
-      hipLaunchKernelGGL(pack_planar_vec, dim3(grid_for(n16, kUnroll)), dim3(256), 0, stream,
+      hipLaunchKernelGGL(pack_planar_vec, dim3(grid_for(n16, kPackPerThread)), dim3(256), 0, stream,
                          reinterpret_cast<const uint4_t *>(in), out, n16);
     }
   } else if (aligned && interleaved && n % 64 == 0) {
