@@ -163,9 +163,10 @@ __global__ __launch_bounds__(256) void unpack_scalar(const unsigned *__restrict_
 }
 
 unsigned grid_for(size_t items, size_t per_thread) {
-  // One 16-byte item per thread and as many blocks as that takes measured
-  // fastest on this part (the streams are read or written exactly once, with
-  // the non-temporal hint); the grid-stride loops only matter beyond the cap.
+  // As many blocks as the items take at `per_thread` items a thread (few items
+  // per thread measured fastest on this part: the streams are read or written
+  // exactly once, with the non-temporal hint); the grid-stride loops only
+  // matter beyond the cap.
   const size_t want = ceil_div(items, 256 * per_thread);
   const size_t cap = (size_t)1 << 30;
   size_t g = want < cap ? want : cap;
