@@ -79,3 +79,67 @@ def test_random_cases(seed):
         if c_axis == INTERLEAVED:
             got = got.reshape(B, rows, cols, 2).transpose(0, 3, 1, 2)
         check_float(got.reshape(w64.shape), dequantize(want, tout).reshape(w64.shape), w64, tin, tout)
+
+
+def _pack_rows(bits, B, rows, K):
+    """One byte per sample [B][2][rows][K] -> rows of whole 32-bit words, LSB first."""
+    kw = (K + 31) // 32
+    padded = np.zeros((B * 2 * rows, kw * 32), dtype=np.uint8)
+    padded[:, :K] = bits.reshape(B * 2 * rows, K)
+    return np.packbits(padded, axis=1, bitorder="little").view(np.uint32).reshape(-1)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_int1_cases(seed, monkeypatch):
+    """1-bit GEMM and pipeline, bit-exact: both variants, ragged shapes, integer alpha / beta,
+    and the switches that select the popcount kernel, a capped workspace (several passes) or
+    a single stream."""
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        B = int(rng.integers(1, 6))
+        M = int(rng.choice([1, 16, 64, 100, 128, 130, 256, 300]))
+        N = int(rng.choice([1, 8, 64, 70, 128, 200, 256, 384]))
+        way = int(rng.integers(4))   # GEMM basic, GEMM opt, pipeline opt, pipeline basic
+        K = (int(rng.choice([32, 64, 96, 512, 992, 1024, 2048, 4096])) if way in (1, 2)
+             else int(rng.choice([1, 31, 32, 33, 100, 512, 1000, 2048, 4097])))
+        if way == 3 and K % 32:
+            K = 32 * (K // 32 + 1)   # the pipeline's flat packing needs rows of whole words
+        c_order = ROW if rng.integers(2) else COL
+        alpha = complex(int(rng.integers(-3, 4)), int(rng.integers(-3, 4)))
+        beta = complex(int(rng.integers(-2, 3)), int(rng.integers(-2, 3))) if rng.integers(2) else 0j
+        switch = int(rng.integers(4))
+        with monkeypatch.context() as env:
+            for name in ("CCGLIB_AMD_INT1_KERNEL", "CCGLIB_AMD_INT1_WORKSPACE_MB", "CCGLIB_AMD_INT1_OVERLAP"):
+                env.delenv(name, raising=False)
+            if switch == 1:
+                env.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
+            elif switch == 2:
+                env.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+            elif switch == 3:
+                env.setenv("CCGLIB_AMD_INT1_OVERLAP", "0")
+            print("seed %d case %d: B=%d M=%d N=%d K=%d way %d C %s alpha=%s beta=%s switch %d" % (
+                seed, case, B, M, N, K, way, "row" if c_order == ROW else "col", alpha, beta, switch),
+                flush=True)
+            a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
+            b_bits = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8)
+            c_in = rng.integers(-1000, 1000, B * 2 * M * N).astype(np.int32)
+            pa, pb = _pack_rows(a_bits, B, M, K), _pack_rows(b_bits, B, N, K)
+            want = orc.gemm(pa, pb, M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, c_in)
+            d_c = to_device(c_in)
+            if way in (0, 1):
+                variant = cc.Variant.opt if way == 1 else cc.Variant.basic
+                gemm = cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.int1, VT.int32), variant, PLANAR,
+                               c_order, ROW, COL, alpha, beta)
+                if way == 1:
+                    d_a, d_b = transpose_operand(pa, B, M, K, VT.int1), transpose_operand(pb, B, N, K, VT.int1)
+                else:
+                    d_a, d_b = to_device(pa), to_device(pb)
+                gemm.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+            else:
+                variant = cc.Variant.opt if way == 2 else cc.Variant.basic
+                pipe = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, c_order, VT.int1,
+                                   VT.int32, variant, alpha, beta)
+                d_a, d_b = to_device(a_bits), to_device(b_bits)
+                pipe.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+            torch.cuda.synchronize()
+            assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
