@@ -367,6 +367,12 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   if (g->K == 0 && g->variant == kOpt) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "K = 0 has no tiled layout");
   }
+  if (g->variant == kOpt && !g->input_interleaved &&
+      ((uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0)) {
+    // tiles are copied to LDS in 16-byte pieces (what Transpose writes into
+    // hipMalloc'ed memory is aligned far beyond this)
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "tiled operands must be 16-byte aligned");
+  }
   DeviceGuard guard(g->device);
   HIP_TRY(guard.status());
   if (g->retile) {

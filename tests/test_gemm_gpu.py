@@ -191,6 +191,22 @@ def test_narrow_planar_c_alpha_only(tin, tout, c_order):
     float_case(2, 256, 516, 64, tin, tout, cc.Variant.basic, PLANAR, c_order, seed=25)   # N % 8 != 0: direct
 
 
+def test_opt_rejects_misaligned_tiles():
+    # tiles go to LDS in 16-byte pieces: a tiled operand that is not 16-byte aligned is an
+    # argument error, not a fault
+    B, M, N, K = 1, 128, 128, 64
+    q = quantize(np.ones(B * 2 * M * K), VT.float16)
+    d_a, d_b = transpose_operand(q, B, M, K, VT.float16), transpose_operand(q, B, N, K, VT.float16)
+    d_c = to_device(np.zeros(B * 2 * M * N, dtype=np.float32))
+    gemm = cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.float16, VT.float32), cc.Variant.opt)
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        gemm.Run(d_a.data_ptr() + 2, d_b.data_ptr(), d_c.data_ptr())
+    gemm.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    c = to_host(d_c, np.float32).reshape(B, 2, M, N)
+    assert np.all(c[:, 0] == 0) and np.all(c[:, 1] == 2 * K)
+
+
 def test_fp32_alpha_beta_and_many_tiles():
     float_case(3, 256, 320, 96, VT.float32, VT.float32, cc.Variant.opt, INTERLEAVED, COL,
                alpha=0.75 - 0.5j, beta=0.5 - 0.25j)
