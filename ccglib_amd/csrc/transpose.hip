@@ -91,12 +91,15 @@ __device__ __forceinline__ void load_ragged(const char *p, size_t plane_stride_b
   im = __builtin_bit_cast(uint4_t, i);
 }
 
-constexpr int kRowsPerThread = 4;
+constexpr int kRowsPerThread = 2;
 constexpr int kVecsPerBlockRow = 16;   // 256 bytes of a row per block
 constexpr int kRowsPerBlock = 16 * kRowsPerThread;
 
-// grid: (ceil(n_vecs_padded / 16), ceil(Mp / 64), B); block: 256 threads as
-// 16 vectors x 16 rows, each thread doing rows r, r+16, r+32, r+48.
+// grid: (ceil(n_vecs_padded / 16), ceil(Mp / 32), B); block: 256 threads as
+// 16 vectors x 16 rows, each thread doing rows r and r+16 (two rows a thread
+// measured best over the operand shapes of the benchmark configurations: one
+// row is as good for 16-bit but slower for 8-bit elements, four are 2-7 %
+// slower, eight halve the rate).
 // RAGGED: input rows of any length at any element-aligned address (the output
 // tiles still hold whole vectors per row).
 template <int EB, bool INTERLEAVED, bool RAGGED>
