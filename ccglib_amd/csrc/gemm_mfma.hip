@@ -294,18 +294,29 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, int x_frag_of
     yi = yi_next;
     yin = negate<DT>(yi);
     CCGLIB_PIN;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc_re[j][i] = mfma<DT>(xr[i], yr, acc_re[j][i]);
+    // from one MFMA to the next only one of the two operands changes (measured 1-2 %
+    // faster on random data than four MFMAs per Y fragment in a row: the part is
+    // power limited, and this order toggles fewer operand bits)
+    acc_re[j][0] = mfma<DT>(xr[0], yr, acc_re[j][0]);
+    acc_im[j][0] = mfma<DT>(xr[0], yi, acc_im[j][0]);
+    acc_im[j][1] = mfma<DT>(xr[1], yi, acc_im[j][1]);
+    acc_re[j][1] = mfma<DT>(xr[1], yr, acc_re[j][1]);
     if (j < 3) yr_next = rd(y_frag_off + (j + 1) * ROW16);
     CCGLIB_PIN;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc_im[j][i] = mfma<DT>(xr[i], yi, acc_im[j][i]);
+    acc_re[j][2] = mfma<DT>(xr[2], yr, acc_re[j][2]);
+    acc_im[j][2] = mfma<DT>(xr[2], yi, acc_im[j][2]);
+    acc_im[j][3] = mfma<DT>(xr[3], yi, acc_im[j][3]);
+    acc_re[j][3] = mfma<DT>(xr[3], yr, acc_re[j][3]);
     if (j < 3) yi_next = rd(y_frag_off + YP + (j + 1) * ROW16);
     CCGLIB_PIN;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc_re[j][i] = mfma<DT>(xi[i], yin, acc_re[j][i]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc_im[j][i] = mfma<DT>(xi[i], yr, acc_im[j][i]);
+    acc_im[j][0] = mfma<DT>(xi[0], yr, acc_im[j][0]);
+    acc_re[j][0] = mfma<DT>(xi[0], yin, acc_re[j][0]);
+    acc_re[j][1] = mfma<DT>(xi[1], yin, acc_re[j][1]);
+    acc_im[j][1] = mfma<DT>(xi[1], yr, acc_im[j][1]);
+    acc_im[j][2] = mfma<DT>(xi[2], yr, acc_im[j][2]);
+    acc_re[j][2] = mfma<DT>(xi[2], yin, acc_re[j][2]);
+    acc_re[j][3] = mfma<DT>(xi[3], yin, acc_re[j][3]);
+    acc_im[j][3] = mfma<DT>(xi[3], yr, acc_im[j][3]);
     CCGLIB_PIN;
   }
 #undef CCGLIB_PIN
@@ -563,10 +574,11 @@ __device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, c
     acc_im[j][0] = mfma<DT>(x[0], y2, acc_im[j][0]);
     if (r == 2 || r == 3) xb[2 * (r - 2)] = rd(x_off[1] + 2 * (r - 2) * ROW16);
     CCGLIB_PIN;
-    acc_re[j][1] = mfma<DT>(x[1], y1, acc_re[j][1]);
+    // (from one MFMA to the next only one of the two operands changes)
+    acc_im[j][1] = mfma<DT>(x[1], y2, acc_im[j][1]);
     if (r == 2 || r == 3) xb[2 * (r - 2) + 1] = rd(x_off[1] + (2 * (r - 2) + 1) * ROW16);
     CCGLIB_PIN;
-    acc_im[j][1] = mfma<DT>(x[1], y2, acc_im[j][1]);
+    acc_re[j][1] = mfma<DT>(x[1], y1, acc_re[j][1]);
     CCGLIB_PIN;
     acc_re[j][2] = mfma<DT>(x[2], y1, acc_re[j][2]);
     if (r + 1 < 8) flip2(y1n, next_raw, 0);
@@ -574,10 +586,10 @@ __device__ __forceinline__ void mma_step_interleaved_ordered(const char *slot, c
     acc_im[j][2] = mfma<DT>(x[2], y2, acc_im[j][2]);
     if (r + 1 < 8) flip2(y1n, next_raw, 2);
     CCGLIB_PIN;
-    acc_re[j][3] = mfma<DT>(x[3], y1, acc_re[j][3]);
+    acc_im[j][3] = mfma<DT>(x[3], y2, acc_im[j][3]);
     if (r + 1 < 8) swap2(y2n, next_raw, 0);
     CCGLIB_PIN;
-    acc_im[j][3] = mfma<DT>(x[3], y2, acc_im[j][3]);
+    acc_re[j][3] = mfma<DT>(x[3], y1, acc_re[j][3]);
     if (r + 1 < 8) swap2(y2n, next_raw, 2);
     CCGLIB_PIN;
     if (r == 0) {
