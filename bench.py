@@ -27,8 +27,8 @@ if ROOT not in sys.path:
 # published dense peaks of MI355X
 MFMA_PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "fp8": 5033.2}
 HBM_PEAK_GBS = 8000.0
-# The 1-bit GEMM runs on the fp4 MFMA (operands expanded to +-1 nibbles by a
-# bandwidth-bound kernel that is part of the GEMM call): published fp4 dense peak
+# The 1-bit GEMM runs on the fp4 MFMA (the packed words are expanded to +-1
+# nibbles in registers, inside the GEMM kernel): published fp4 dense peak
 FP4_PEAK_TOPS = 10066.3
 
 WORKLOADS = {
@@ -247,7 +247,7 @@ def main():
 
     if tin == VT.int1:
         dtype, peak, bound, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "mfma", "TOP/s"
-        kernel_name = "expand_int1_to_fp4 x2 + complex_gemm_mfma_dtl<fp4->int32>"
+        kernel_name = "complex_gemm_mfma_dtl<int1->int32> (fp4 MFMA, bits expanded in registers)"
     else:
         dtype = {"float16": "f16", "bfloat16": "bf16"}.get(tin_name, "fp8")
         peak, bound, unit = MFMA_PEAK_TFLOPS[dtype], "mfma", "TFLOP/s"
@@ -308,8 +308,8 @@ def main():
             "max_abs_diff_vs_unfused": float((c2 - c).abs().max())}
 
     if tin == VT.int1:
-        # The same job through Pipeline.Run, which expands the one-byte-per-sample input
-        # straight into the 1-bit GEMM's workspace (no packed or transposed intermediates).
+        # The same job through Pipeline.Run, which packs the one-byte-per-sample input
+        # straight into the tiled 1-bit layout (no packed, untransposed intermediate).
         c2 = torch.empty_like(c)
         pipe = cc.Pipeline(B, M, N, K, 0, stream, AX.complex_planar, AX.complex_planar,
                            MO.row_major, MO.col_major, MO.row_major, tin, tout, cc.Variant.opt)

@@ -115,6 +115,8 @@ struct ccglib_gemm {
   // retile_b_offset) and the kernel of the opt variant runs on the copies.
   bool retile = false;
   size_t retile_b_offset = 0;
+  // 1-bit GEMM: the MFMA kernel may read the packed words as they are
+  int int1_direct = 1;
 };
 
 struct ccglib_transpose {
@@ -214,6 +216,7 @@ void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, vo
   p.workspace = g->workspace;
   p.workspace_bytes = g->workspace_bytes;
   p.aux = g->aux.stream ? &g->aux : nullptr;
+  p.int1_direct = g->int1_direct;
 }
 
 }  // namespace
@@ -295,11 +298,15 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
   g->beta_re = beta_re;
   g->beta_im = beta_im;
   if (type_in == kInt1 && B && M && N) {
-    // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs;
+    // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs,
+    // =expand on the MFMA kernel that reads an fp4 copy of the operands (the one
+    // used anyway for planar rows that are not whole 16-byte chunks);
     // CCGLIB_AMD_INT1_WORKSPACE_MB caps the expanded operands (the GEMM then runs
     // in groups of batches). Failing to get the memory is not an error.
     const char *kernel = std::getenv("CCGLIB_AMD_INT1_KERNEL");
     const char *cap_mb = std::getenv("CCGLIB_AMD_INT1_WORKSPACE_MB");
+    g->int1_direct = !(kernel && (std::strcmp(kernel, "popcount") == 0 ||
+                                  std::strcmp(kernel, "expand") == 0));
     size_t bytes = gemm_int1_workspace_bytes(B, M, N, K);
     const size_t per_batch = bytes / B;
     size_t cap = cap_mb ? (size_t)std::strtoull(cap_mb, nullptr, 10) << 20 : (size_t)16 << 30;

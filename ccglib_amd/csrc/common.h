@@ -92,6 +92,9 @@ struct GemmParams {
   // 1-bit GEMM only: where the expansion of later batches may run while earlier
   // batches are multiplied (may be null: everything on the one stream)
   const GemmAux *aux = nullptr;
+  // 1-bit GEMM only: the MFMA kernel may take the packed words as they are
+  // (no expanded copy) when their layout allows it
+  int int1_direct = 1;
 };
 
 // Bytes of workspace with which the 1-bit GEMM of this size runs in one pass.

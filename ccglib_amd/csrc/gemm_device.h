@@ -99,6 +99,8 @@ struct KernelArgs {
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta, c_interleaved;
   int c_vector_ok;  // C base is 16-byte aligned: wide stores allowed
+  // 1-bit samples on the MFMA: what the zero bits past K add to every imaginary sum
+  unsigned im_excess;
 };
 
 // Maps the hardware workgroup id to a logical tile id such that the ids that
@@ -171,6 +173,7 @@ inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
   a.have_beta = p.have_beta;
   a.c_interleaved = p.c_interleaved;
   a.c_vector_ok = ((uintptr_t)p.c % 16 == 0);
+  a.im_excess = (p.type_in == kInt1) ? 2u * (p.k_tiles * (unsigned)k_per_tile(kInt1) - p.k) : 0u;
   return a;
 }
 

@@ -335,6 +335,71 @@ __global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *
   }
 }
 
+// One byte per sample straight into the tiled 1-bit layout that the opt variant
+// reads ([batch][rows/128][K/512][2][128 rows][64 bytes]; rows and samples past
+// the end are zero bits): Packing and Transpose of the reference's pipeline
+// (src/pipeline/Pipeline.cpp:111-121) in one pass without the packed intermediate.
+// A wave takes 16 rows of a tile, four at a time: lane = (row of the four, 16-byte
+// piece p of 256 bytes), and two load instructions cover the 512 samples of a tile
+// row, each reading four runs of 256 contiguous bytes; a thread has eight loads in
+// flight. A thread's 16 bytes are half an output word: lane pairs exchange one
+// half each, after which the even lane holds word p / 2 of the row (from the first
+// 256 samples) and the odd lane word 8 + p / 2 (from the second), so that a store
+// instruction of a wave writes four whole tile rows, 256 contiguous bytes.
+template <bool VEC>
+__global__ __launch_bounds__(256) void pack_bytes_to_tiles(const unsigned char *__restrict__ src,
+                                                           char *__restrict__ dst, unsigned rows,
+                                                           unsigned row_tiles, unsigned k,
+                                                           unsigned k1_tiles) {
+  // blockIdx: x = K tile of 512 samples, y = block of 64 rows, z = (batch, plane)
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned p = lane & 15;
+  const unsigned rt = blockIdx.y >> 1;
+  const size_t b = blockIdx.z >> 1;
+  const unsigned plane = blockIdx.z & 1;
+  const unsigned k_base = blockIdx.x * 512 + p * 16;
+  unsigned row_in_tile[4], n[4][2];
+  const unsigned char *row_ptr[4];
+  uint4_t v[4][2];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    row_in_tile[q] = (blockIdx.y & 1) * 64 + wave * 16 + q * 4 + (lane >> 4);
+    const unsigned r = rt * kTileRows + row_in_tile[q];
+    row_ptr[q] = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const unsigned k0 = k_base + h * 256;
+      n[q][h] = (r < rows && k0 < k) ? (k - k0 < 16 ? k - k0 : 16) : 0;
+      if (VEC && n[q][h] == 16) {
+        v[q][h] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0));
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned half[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (VEC && n[q][h] == 16) {
+        half[h] = nonzero_bits_of16(v[q][h]);
+      } else {
+        half[h] = 0;
+        const unsigned k0 = k_base + h * 256;
+        for (unsigned i = 0; i < n[q][h]; ++i) half[h] |= (row_ptr[q][k0 + i] != 0 ? 1u : 0u) << i;
+      }
+    }
+    // the neighbour (lane ^ 1) gets the half this lane does not keep
+    const bool odd = (lane & 1) != 0;
+    const unsigned give = odd ? half[0] : half[1];
+    const unsigned got = (unsigned)__builtin_amdgcn_update_dpp(0, (int)give, 0xB1, 0xf, 0xf, false);
+    const unsigned word = odd ? (got | (half[1] << 16)) : (half[0] | (got << 16));
+    const unsigned word_index = (p >> 1) + (odd ? 8 : 0);
+    *reinterpret_cast<unsigned *>(dst + ((b * row_tiles + rt) * k1_tiles + blockIdx.x) * kTileBytes +
+                                  plane * kTilePlaneBytes + row_in_tile[q] * kTileRowBytes +
+                                  4 * word_index) = word;
+  }
+}
+
 // Largest K for which every partial sum (at most 2 K in magnitude) is exact in fp32.
 constexpr unsigned kMaxMfmaK = 1u << 22;
 
@@ -396,8 +461,23 @@ hipError_t run_groups(const GemmParams &p, hipStream_t stream, size_t group, boo
   return hipGetLastError();
 }
 
+// The packed words as they are: tiled operands always (16-byte aligned, which
+// the caller has checked), planar rows when they are whole aligned 16-byte
+// chunks (K a multiple of 128).
+bool direct_ok(const GemmParams &p) {
+  if (!p.int1_direct || p.k == 0 || p.k > kMaxMfmaK || p.input_interleaved) return false;
+  if (((uintptr_t)p.x | (uintptr_t)p.y) % 16 != 0) return false;
+  if (p.variant == kOpt) return true;
+  const size_t k_bytes = ceil_div(p.k, 32) * 4;
+  return k_bytes % 16 == 0;
+}
+
 hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *done) {
   *done = false;
+  if (direct_ok(p)) {
+    *done = true;
+    return launch_gemm_mfma(p, stream);
+  }
   if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
   const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
   const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
@@ -447,6 +527,33 @@ bool gemm_int1_can_take_bytes(const GemmParams &p) {
 
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
   if (!gemm_int1_can_take_bytes(p)) return hipErrorInvalidValue;
+  if (p.int1_direct) {
+    // pack into the tiled 1-bit layout (a quarter of the workspace) and multiply
+    // the packed words as they are
+    const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
+    const size_t x_bytes = (size_t)p.batch * p.x_tiles * k1_tiles * kTileBytes;
+    char *ws_x = static_cast<char *>(p.workspace), *ws_y = ws_x + x_bytes;
+    for (int which = 0; which < 2; ++which) {
+      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+      const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
+      const dim3 grid(k1_tiles, 2 * row_tiles, 2 * p.batch);
+      const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
+      if (vec) {
+        hipLaunchKernelGGL(pack_bytes_to_tiles<true>, grid, dim3(256), 0, stream, src,
+                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
+      } else {
+        hipLaunchKernelGGL(pack_bytes_to_tiles<false>, grid, dim3(256), 0, stream, src,
+                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
+      }
+    }
+    if (hipError_t e = hipGetLastError()) return e;
+    GemmParams q = p;
+    q.x = ws_x;
+    q.y = ws_y;
+    q.variant = kOpt;
+    q.k_tiles = k1_tiles;
+    return launch_gemm_mfma(q, stream);
+  }
   const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
   auto expand = [&](size_t b0, size_t nb, char *ws_x, char *ws_y, hipStream_t s) -> hipError_t {
     for (int which = 0; which < 2; ++which) {

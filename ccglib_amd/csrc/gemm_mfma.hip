@@ -453,6 +453,142 @@ __device__ __forceinline__ void mma_step32_ordered(const char *slot, const int (
 #undef CCGLIB_PIN
 }
 
+// 1-bit samples, multiplied on the fp4 MFMA straight from the packed words.
+// A 64-byte row of a slot holds 512 samples; a lane reads its two 16-byte
+// chunks of a row as for the other 32-row MFMAs, and each of the eight words
+// it then holds feeds one 32x32x64 MFMA (64 samples of K: 32 from each half of
+// the wave). A word becomes the MFMA's four operand registers with seven
+// vector-ALU instructions: nibble i of register j is 0x2 | bit (4 i + j) << 3,
+// i.e. fp4 +1.0 for a 0 bit and -1.0 for a 1 bit. Which sample lands in which
+// K position of the instruction does not matter as long as X and Y agree, and
+// neither does the sign convention (bit 1 = +1 in src/reference/GEMM.cpp:131-200):
+// negating X and Y together leaves every product as it is. The expansion of the
+// fragment that is needed two to four MFMAs later is placed behind each MFMA,
+// in whose shadow the vector ALU is otherwise idle; the MFMAs are issued so
+// that only one operand changes from one to the next.
+// Samples past K (zero bits in both operands, which the tiled layout and the
+// zero tile guarantee) add 0 to every real and +2 to every imaginary sum; the
+// epilogue takes that off (KernelArgs::im_excess), which is the reference's
+// K_PADDING correction (kernels/gemm_kernel_int1.cu:64-196).
+__device__ __forceinline__ int4_t expand_bits(int word) {
+  const unsigned w = (unsigned)word;
+  int4_t o;
+  // (a & b) | c in one instruction (truth table 0xEA)
+  o[0] = (int)__builtin_amdgcn_bitop3_b32(w << 3, 0x88888888u, 0x22222222u, 0xEA);
+  o[1] = (int)__builtin_amdgcn_bitop3_b32(w << 2, 0x88888888u, 0x22222222u, 0xEA);
+  o[2] = (int)__builtin_amdgcn_bitop3_b32(w << 1, 0x88888888u, 0x22222222u, 0xEA);
+  o[3] = (int)__builtin_amdgcn_bitop3_b32(w, 0x88888888u, 0x22222222u, 0xEA);
+  return o;
+}
+
+__device__ __forceinline__ float16_t_ mfma_fp4(const int4_t &a, const int4_t &b, float16_t_ acc) {
+  // format code 4 = fp4 (only the low four registers are read); scale 2^0
+  const int8_t_ av = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+  const int8_t_ bv = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 0, 0x7f, 0, 0x7f);
+}
+
+template <int BX, int BY, typename Mid>
+__device__ __forceinline__ void mma_step32_bits(const char *slot, const int (&x_off)[2],
+                                                const int (&y_off)[2], float16_t_ (&acc_re)[2][2],
+                                                float16_t_ (&acc_im)[2][2], Mid &&mid) {
+  constexpr int ROW32 = 32 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
+  // fragments: 0 x0r, 1 x0i, 2 x1r, 3 x1i, 4 y0r, 5 y0i, 6 y1r, 7 y1i
+  enum { X0R, X0I, X1R, X1I, Y0R, Y0I, Y1R, Y1I };
+  int4_t raw[8];    // the chunk (four words, one per MFMA step) in use
+  auto rd = [&](int f, int u) {
+    const int off = (f < 4 ? x_off[u] : y_off[u]) + ((f & 1) ? (f < 4 ? XP : YP) : 0) +
+                    ((f & 2) ? ROW32 : 0);
+    raw[f] = *reinterpret_cast<const int4_t *>(slot + off);
+  };
+  auto neg = [](const int4_t &f) {
+    int4_t r;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r[w] = f[w] ^ (int)0x88888888u;
+    return r;
+  };
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+  // in order of first use
+  rd(X0R, 0);
+  rd(Y0R, 0);
+  rd(Y0I, 0);
+  rd(Y1I, 0);
+  rd(Y1R, 0);
+  rd(X1R, 0);
+  rd(X1I, 0);
+  rd(X0I, 0);
+  CCGLIB_PIN;
+  int4_t x0r = expand_bits(raw[X0R][0]), y0r = expand_bits(raw[Y0R][0]),
+         y0i = expand_bits(raw[Y0I][0]);
+  int4_t x0i, x1r, x1i, y1r, y1i, y0n, y1n, x0r_next, y0r_next, y0i_next;
+  CCGLIB_PIN;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const int w = s & 3;
+    // after a chunk's last word has been taken, the next chunk of the row is read
+    // into the same registers (its first word is needed sixteen MFMAs later)
+    const bool reload = (s == 3);
+    const bool reload_next = (s == 2);   // for the fragments expanded one step ahead
+    acc_re[0][0] = mfma_fp4(x0r, y0r, acc_re[0][0]);
+    y1i = expand_bits(raw[Y1I][w]);
+    if (reload) rd(Y1I, 1);
+    CCGLIB_PIN;
+    acc_im[0][0] = mfma_fp4(x0r, y0i, acc_im[0][0]);
+    y1r = expand_bits(raw[Y1R][w]);
+    if (reload) rd(Y1R, 1);
+    CCGLIB_PIN;
+    acc_im[1][0] = mfma_fp4(x0r, y1i, acc_im[1][0]);
+    x1r = expand_bits(raw[X1R][w]);
+    if (reload) rd(X1R, 1);
+    CCGLIB_PIN;
+    acc_re[1][0] = mfma_fp4(x0r, y1r, acc_re[1][0]);
+    x1i = expand_bits(raw[X1I][w]);
+    if (reload) rd(X1I, 1);
+    CCGLIB_PIN;
+    if (s == 0) {
+      mid();
+      CCGLIB_PIN;
+    }
+    acc_re[1][1] = mfma_fp4(x1r, y1r, acc_re[1][1]);
+    y0n = neg(y0i);
+    CCGLIB_PIN;
+    acc_im[1][1] = mfma_fp4(x1r, y1i, acc_im[1][1]);
+    y1n = neg(y1i);
+    CCGLIB_PIN;
+    acc_im[0][1] = mfma_fp4(x1r, y0i, acc_im[0][1]);
+    x0i = expand_bits(raw[X0I][w]);
+    if (reload) rd(X0I, 1);
+    CCGLIB_PIN;
+    acc_re[0][1] = mfma_fp4(x1r, y0r, acc_re[0][1]);
+    CCGLIB_PIN;
+    acc_im[0][1] = mfma_fp4(x1i, y0r, acc_im[0][1]);
+    CCGLIB_PIN;
+    acc_re[0][1] = mfma_fp4(x1i, y0n, acc_re[0][1]);
+    if (s < 7) x0r_next = expand_bits(raw[X0R][(s + 1) & 3]);
+    if (reload_next) rd(X0R, 1);
+    CCGLIB_PIN;
+    acc_re[1][1] = mfma_fp4(x1i, y1n, acc_re[1][1]);
+    if (s < 7) y0r_next = expand_bits(raw[Y0R][(s + 1) & 3]);
+    if (reload_next) rd(Y0R, 1);
+    CCGLIB_PIN;
+    acc_im[1][1] = mfma_fp4(x1i, y1r, acc_im[1][1]);
+    if (s < 7) y0i_next = expand_bits(raw[Y0I][(s + 1) & 3]);
+    if (reload_next) rd(Y0I, 1);
+    CCGLIB_PIN;
+    acc_im[1][0] = mfma_fp4(x0i, y1r, acc_im[1][0]);
+    acc_re[1][0] = mfma_fp4(x0i, y1n, acc_re[1][0]);
+    acc_re[0][0] = mfma_fp4(x0i, y0n, acc_re[0][0]);
+    acc_im[0][0] = mfma_fp4(x0i, y0r, acc_im[0][0]);
+    CCGLIB_PIN;
+    if (s < 7) {
+      x0r = x0r_next;
+      y0r = y0r_next;
+      y0i = y0i_next;
+    }
+  }
+#undef CCGLIB_PIN
+}
+
 // The same for interleaved operands (rows of (re, im) pairs, as the caller's
 // buffers hold them). With K running over the 2K real numbers of a row,
 //   Re = sum X~ . Y1,  Y1 = (yr, -yi, ...)   and   Im = sum X~ . Y2,  Y2 = (yi, yr, ...)
@@ -807,7 +943,7 @@ __device__ __forceinline__ void store_wave_tile_int32(const KernelArgs &args, un
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const unsigned sr = (unsigned)(int)piece_elem<MS>(acc_re, j, i, e);
-        const unsigned si = (unsigned)(int)piece_elem<MS>(acc_im, j, i, e);
+        const unsigned si = (unsigned)(int)piece_elem<MS>(acc_im, j, i, e) - args.im_excess;
         re[e] = ar * sr - ai * si;
         im[e] = ai * sr + ar * si;
       }
@@ -1021,7 +1157,7 @@ __device__ __forceinline__ void store_wave_tile_staged32(const KernelArgs &args,
             const float re = acc_re[j][i][4 * k + e], im = acc_im[j][i][4 * k + e];
             if constexpr (INT) {
               // exact integers; alpha truncated, arithmetic modulo 2^32
-              const unsigned sr = (unsigned)(int)re, si = (unsigned)(int)im;
+              const unsigned sr = (unsigned)(int)re, si = (unsigned)(int)im - args.im_excess;
               const unsigned iar = (unsigned)(int)ar, iai = (unsigned)(int)ai;
               const unsigned o = plane == 0 ? iar * sr - iai * si : iai * sr + iar * si;
               v[e] = __builtin_bit_cast(float, o);
@@ -1458,7 +1594,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         const char *tile[KPM];
 #pragma unroll
         for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
-        if constexpr (MS == 32 && TX == 2 && TY == 2) {
+        if constexpr (DT == kInt1) {
+          static_assert(MS == 32 && TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
+          mma_step32_bits<BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+        } else if constexpr (MS == 32 && TX == 2 && TY == 2) {
           mma_step32_ordered<DT, BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
         } else if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
@@ -1675,6 +1814,15 @@ hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
       break;
     case kFloat8e5m2:
       if (p.type_out == kFloat32) return launch_typed<kFloat8e5m2, kFloat32>(p, stream);
+      break;
+    case kInt1:
+      // packed 1-bit samples expanded in registers; the caller has checked that
+      // planar rows are whole aligned 16-byte chunks and that K fits fp32 sums
+      if (p.type_out == kInt32 && !p.input_interleaved) {
+        return p.variant == kOpt
+                   ? launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
+                   : launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
+      }
       break;
     case kFp4Sign:
       // the 1-bit GEMM's operands expanded to fp4 +-1, tiled; exact integer sums

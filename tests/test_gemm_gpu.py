@@ -281,19 +281,24 @@ def test_batches_are_independent():
 
 # ---- 1-bit ------------------------------------------------------------------------------
 
-@pytest.fixture(params=["mfma", "mfma_grouped", "popcount"])
+@pytest.fixture(params=["mfma", "expand", "expand_grouped", "popcount"])
 def int1_kernel(request, monkeypatch):
-    """The 1-bit GEMM has two implementations behind one entry point: fp4 MFMA on
-    expanded operands (default; "grouped" = a workspace cap that forces several
-    passes over groups of batches) and XOR + popcount on the vector ALUs (used
-    when K is too large for exact fp32 sums or the workspace cannot be had). The
-    choice is read from the environment when the GEMM object is created."""
+    """The 1-bit GEMM has three implementations behind one entry point: the fp4 MFMA
+    kernel that expands the packed words in registers (default, where the layout
+    allows it: tiled operands, or planar rows of whole 16-byte chunks), the same
+    MFMA on an expanded copy of the operands ("expand"; "grouped" = a workspace cap
+    that forces several passes over groups of batches) and XOR + popcount on the
+    vector ALUs (used when K is too large for exact fp32 sums or the workspace
+    cannot be had). The choice is read from the environment when the GEMM object is
+    created."""
     monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
     monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
     if request.param == "popcount":
         monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
-    elif request.param == "mfma_grouped":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+    elif request.param.startswith("expand"):
+        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
+        if request.param == "expand_grouped":
+            monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
     return request.param
 
 

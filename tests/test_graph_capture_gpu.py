@@ -37,6 +37,7 @@ def _capture_and_replay(make_object, inputs, fill_inputs, out_shape, out_dtype, 
         torch.cuda.synchronize()
         got = d_c.clone()
         d_c.zero_()
+        torch.cuda.synchronize()            # `side` does not wait for the stream zero_() ran on
         with torch.cuda.stream(side):
             obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
         torch.cuda.synchronize()

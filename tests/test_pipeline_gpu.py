@@ -102,17 +102,20 @@ def test_pipeline_int1(variant):
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
-@pytest.mark.parametrize("mode", ["direct", "popcount", "capped_workspace"])
+@pytest.mark.parametrize("mode", ["direct", "expand", "popcount", "capped_workspace"])
 @pytest.mark.parametrize("M,N,K,c_order", [(130, 70, 992, ROW), (64, 200, 96, COL), (20, 30, 32, ROW),
                                            (256, 128, 2048, COL)])
 def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
-    # Planar one-byte-per-sample input is expanded straight into the 1-bit GEMM's
-    # workspace ("direct"); without a (whole) workspace the pipeline packs and
-    # transposes as the reference does. Any non-zero byte is a 1 bit.
+    # Planar one-byte-per-sample input is packed straight into the tiled 1-bit layout
+    # in the GEMM's workspace ("direct") or expanded into fp4 values there ("expand");
+    # without a (whole) workspace the pipeline packs and transposes as the reference
+    # does. Any non-zero byte is a 1 bit.
     monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
     monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
     if mode == "popcount":
         monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
+    elif mode == "expand":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
     elif mode == "capped_workspace":
         monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
     B = 3
@@ -152,6 +155,9 @@ def test_int1_expansion_in_groups(what, overlap, monkeypatch):
     multiply in two groups of 8 batches, the expansion on a second stream (or, with
     CCGLIB_AMD_INT1_OVERLAP=0, everything on the caller's stream). Two Runs in a row with
     different input: the second call's expansion must not overtake the first call's GEMMs."""
+    # (the MFMA kernel on an fp4 copy of the operands; by default the packed words
+    # are multiplied as they are and nothing is expanded)
+    monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
     if not overlap:
         monkeypatch.setenv("CCGLIB_AMD_INT1_OVERLAP", "0")
     B, M, N, K = 16, 1024, 1024, 256
