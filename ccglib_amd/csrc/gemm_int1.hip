@@ -339,64 +339,85 @@ __global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *
 // reads ([batch][rows/128][K/512][2][128 rows][64 bytes]; rows and samples past
 // the end are zero bits): Packing and Transpose of the reference's pipeline
 // (src/pipeline/Pipeline.cpp:111-121) in one pass without the packed intermediate.
-// A wave takes 16 rows of a tile, four at a time: lane = (row of the four, 16-byte
-// piece p of 256 bytes), and two load instructions cover the 512 samples of a tile
-// row, each reading four runs of 256 contiguous bytes; a thread has eight loads in
-// flight. A thread's 16 bytes are half an output word: lane pairs exchange one
-// half each, after which the even lane holds word p / 2 of the row (from the first
-// 256 samples) and the odd lane word 8 + p / 2 (from the second), so that a store
-// instruction of a wave writes four whole tile rows, 256 contiguous bytes.
+// A wave takes 16 rows of a tile, two at a time: lane = (row of the two, 16-byte
+// piece p of the 512 samples of a tile row), so that a load instruction reads two
+// runs of 512 contiguous bytes; a thread has eight loads in flight. A thread's
+// 16 bytes are half an output word: of every two loads, lane pairs exchange one
+// half, after which the even lane holds word p / 2 of the first load's row and
+// the odd lane that of the second's, so that a store instruction of a wave
+// writes four whole tile rows, 256 contiguous bytes.
+// Inside a half word the 16 samples are stored transposed (sample 4 d + j at bit
+// 4 j + d), which saves the bit gathering per 4 bytes: both operands of the GEMM
+// are packed by this kernel, and a sum over K does not see a permutation of K
+// that is the same in X and Y.
+__device__ __forceinline__ unsigned nonzero_bits_transposed(uint4_t v) {
+  unsigned c = 0;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned nz = (((v[d] & 0x7f7f7f7fu) + 0x7f7f7f7fu) | v[d]) & 0x80808080u;
+    c |= nz >> (7 - d);
+  }
+  // byte j of c holds samples j, 4 + j, 8 + j, 12 + j in its low four bits
+  const unsigned t = c | (c >> 4);
+  return (t & 0xffu) | ((t >> 8) & 0xff00u);
+}
+
+constexpr int kPackLoads = 4;   // loads in flight per thread (two rows each per wave)
 template <bool VEC>
 __global__ __launch_bounds__(256) void pack_bytes_to_tiles(const unsigned char *__restrict__ src,
                                                            char *__restrict__ dst, unsigned rows,
                                                            unsigned row_tiles, unsigned k,
                                                            unsigned k1_tiles) {
-  // blockIdx: x = K tile of 512 samples, y = block of 64 rows, z = (batch, plane)
-  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const unsigned p = lane & 15;
-  const unsigned rt = blockIdx.y >> 1;
+  // blockIdx: x = four K tiles of 512 samples (one per wave: a block reads 2 KiB
+  // contiguous of each of its rows), y = block of 2 kPackLoads rows, z = (batch, plane)
+  const unsigned lane = threadIdx.x & 63;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const unsigned p = lane & 31;                 // 16-byte piece of the 512 samples of a tile row
+  constexpr unsigned RPW = 2 * kPackLoads, WPT = kTileRows / RPW;   // rows per wave, waves per tile
+  const unsigned rt = blockIdx.y / WPT;
   const size_t b = blockIdx.z >> 1;
   const unsigned plane = blockIdx.z & 1;
-  const unsigned k_base = blockIdx.x * 512 + p * 16;
-  unsigned row_in_tile[4], n[4][2];
-  const unsigned char *row_ptr[4];
-  uint4_t v[4][2];
+  const unsigned kt = blockIdx.x * 4 + wave;
+  if (kt >= k1_tiles) return;
+  const unsigned k0 = kt * 512 + p * 16;
+  const unsigned row0_in_tile = (blockIdx.y % WPT) * RPW + (lane >> 5);   // + 2 i
+  const unsigned block_row0 = rt * kTileRows + (blockIdx.y % WPT) * RPW;
+  unsigned half[kPackLoads];
+  // the same for all threads of a wave: all its rows and all 512 samples exist
+  if (VEC && block_row0 + RPW <= rows && kt * 512 + 512 <= k) {
+    const unsigned char *p0 =
+        src + ((b * 2 + plane) * rows + rt * kTileRows + row0_in_tile) * (size_t)k + k0;
+    uint4_t v[kPackLoads];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    row_in_tile[q] = (blockIdx.y & 1) * 64 + wave * 16 + q * 4 + (lane >> 4);
-    const unsigned r = rt * kTileRows + row_in_tile[q];
-    row_ptr[q] = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
+    for (int i = 0; i < kPackLoads; ++i) {
+      v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p0 + (size_t)(2 * i) * k));
+    }
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const unsigned k0 = k_base + h * 256;
-      n[q][h] = (r < rows && k0 < k) ? (k - k0 < 16 ? k - k0 : 16) : 0;
-      if (VEC && n[q][h] == 16) {
-        v[q][h] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0));
+    for (int i = 0; i < kPackLoads; ++i) half[i] = nonzero_bits_transposed(v[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < kPackLoads; ++i) {
+      const unsigned r = rt * kTileRows + row0_in_tile + 2 * i;
+      const unsigned char *row_ptr = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
+      const unsigned n = (r < rows && k0 < k) ? (k - k0 < 16 ? k - k0 : 16) : 0;
+      unsigned bits = 0;
+      for (unsigned e = 0; e < n; ++e) {
+        bits |= (row_ptr[k0 + e] != 0 ? 1u : 0u) << (4 * (e & 3) + (e >> 2));
       }
+      half[i] = bits;
     }
   }
+  // Lane pairs hold the two halves of word p / 2 of each row: of every two rows
+  // the even lane takes the word of the first and the odd lane that of the second.
+  const bool odd = (lane & 1) != 0;
+  char *out = dst + ((b * row_tiles + rt) * k1_tiles + kt) * kTileBytes +
+              plane * kTilePlaneBytes + (row0_in_tile + (odd ? 2 : 0)) * kTileRowBytes + 4 * (p >> 1);
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    unsigned half[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if (VEC && n[q][h] == 16) {
-        half[h] = nonzero_bits_of16(v[q][h]);
-      } else {
-        half[h] = 0;
-        const unsigned k0 = k_base + h * 256;
-        for (unsigned i = 0; i < n[q][h]; ++i) half[h] |= (row_ptr[q][k0 + i] != 0 ? 1u : 0u) << i;
-      }
-    }
-    // the neighbour (lane ^ 1) gets the half this lane does not keep
-    const bool odd = (lane & 1) != 0;
-    const unsigned give = odd ? half[0] : half[1];
+  for (int m = 0; m < kPackLoads / 2; ++m) {
+    const unsigned give = odd ? half[2 * m] : half[2 * m + 1];
     const unsigned got = (unsigned)__builtin_amdgcn_update_dpp(0, (int)give, 0xB1, 0xf, 0xf, false);
-    const unsigned word = odd ? (got | (half[1] << 16)) : (half[0] | (got << 16));
-    const unsigned word_index = (p >> 1) + (odd ? 8 : 0);
-    *reinterpret_cast<unsigned *>(dst + ((b * row_tiles + rt) * k1_tiles + blockIdx.x) * kTileBytes +
-                                  plane * kTilePlaneBytes + row_in_tile[q] * kTileRowBytes +
-                                  4 * word_index) = word;
+    const unsigned word = odd ? (got | (half[2 * m + 1] << 16)) : (half[2 * m] | (got << 16));
+    *reinterpret_cast<unsigned *>(out + 4 * m * kTileRowBytes) = word;
   }
 }
 
@@ -522,7 +543,7 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
 bool gemm_int1_can_take_bytes(const GemmParams &p) {
   if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return false;
   if (p.workspace_bytes < gemm_int1_workspace_bytes(p.batch, p.nx, p.ny, p.k)) return false;
-  return p.batch <= 32767 && 2 * (size_t)p.x_tiles <= 65535 && 2 * (size_t)p.y_tiles <= 65535;
+  return p.batch <= 32767 && 16 * (size_t)p.x_tiles <= 65535 && 16 * (size_t)p.y_tiles <= 65535;
 }
 
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
@@ -536,7 +557,7 @@ hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) 
     for (int which = 0; which < 2; ++which) {
       const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
       const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
-      const dim3 grid(k1_tiles, 2 * row_tiles, 2 * p.batch);
+      const dim3 grid((unsigned)ceil_div(k1_tiles, 4), (kTileRows / (2 * kPackLoads)) * row_tiles, 2 * p.batch);
       const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
       if (vec) {
         hipLaunchKernelGGL(pack_bytes_to_tiles<true>, grid, dim3(256), 0, stream, src,
