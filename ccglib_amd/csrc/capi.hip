@@ -177,6 +177,12 @@ void release_aux(GemmAux *aux) {
   aux->stream = nullptr;
 }
 
+// Largest workspace a 1-bit GEMM object allocates (CCGLIB_AMD_INT1_WORKSPACE_MB, default 16 GiB).
+size_t int1_workspace_cap() {
+  const char *cap_mb = std::getenv("CCGLIB_AMD_INT1_WORKSPACE_MB");
+  return cap_mb ? (size_t)std::strtoull(cap_mb, nullptr, 10) << 20 : (size_t)16 << 30;
+}
+
 // Launch parameters of a GEMM object for the given buffers.
 void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, void *d_c,
                       GemmParams *out) {
@@ -299,20 +305,21 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
   g->beta_im = beta_im;
   if (type_in == kInt1 && B && M && N) {
     // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs,
-    // =expand on the MFMA kernel that reads an fp4 copy of the operands (the one
-    // used anyway for planar rows that are not whole 16-byte chunks);
-    // CCGLIB_AMD_INT1_WORKSPACE_MB caps the expanded operands (the GEMM then runs
-    // in groups of batches). Failing to get the memory is not an error.
+    // =expand on the MFMA kernel that reads an fp4 copy of the operands;
+    // CCGLIB_AMD_INT1_WORKSPACE_MB caps that copy (the GEMM then runs in groups
+    // of batches). Failing to get the memory is not an error.
     const char *kernel = std::getenv("CCGLIB_AMD_INT1_KERNEL");
-    const char *cap_mb = std::getenv("CCGLIB_AMD_INT1_WORKSPACE_MB");
-    g->int1_direct = !(kernel && (std::strcmp(kernel, "popcount") == 0 ||
-                                  std::strcmp(kernel, "expand") == 0));
-    size_t bytes = gemm_int1_workspace_bytes(B, M, N, K);
+    const bool popcount = kernel && std::strcmp(kernel, "popcount") == 0;
+    g->int1_direct = !(popcount || (kernel && std::strcmp(kernel, "expand") == 0));
+    // The default kernel multiplies the packed words as they are and needs no
+    // copy; only planar rows that are not whole 16-byte chunks go through one.
+    const bool rows_direct = variant == kOpt || (ceil_div(K, 32) * 4) % 16 == 0;
+    size_t bytes = (g->int1_direct && rows_direct) ? 0 : gemm_int1_workspace_bytes(B, M, N, K);
     const size_t per_batch = bytes / B;
-    size_t cap = cap_mb ? (size_t)std::strtoull(cap_mb, nullptr, 10) << 20 : (size_t)16 << 30;
+    size_t cap = int1_workspace_cap();
     if (cap < per_batch) cap = per_batch;
     if (bytes > cap) bytes = cap / per_batch * per_batch;
-    if (bytes && !(kernel && std::strcmp(kernel, "popcount") == 0)) {
+    if (bytes && !popcount) {
       DeviceGuard guard(device);
       if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes) == hipSuccess) {
         g->workspace_bytes = bytes;
@@ -712,6 +719,19 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
                               kOpt, output_complex_axis_location, c_mem_order, a_mem_order,
                               b_mem_order, alpha_re, alpha_im, beta_re, beta_im);
       if (rc != CCGLIB_OK) break;
+      if (p->gemm->int1_direct && !p->gemm->workspace) {
+        // room for the 1-bit tiles that the caller's bytes are packed into (the
+        // GEMM object owns and frees it)
+        const size_t bytes = gemm_int1_tiles_bytes(B, M, N, K);
+        DeviceGuard guard(device);
+        if (bytes && bytes <= int1_workspace_cap() && guard.status() == hipSuccess &&
+            hipMalloc(&p->gemm->workspace, bytes) == hipSuccess) {
+          p->gemm->workspace_bytes = bytes;
+        } else {
+          p->gemm->workspace = nullptr;
+          (void)hipGetLastError();
+        }
+      }
       GemmParams probe;
       fill_gemm_params(p->gemm, nullptr, nullptr, nullptr, &probe);
       if (gemm_int1_can_take_bytes(probe)) {

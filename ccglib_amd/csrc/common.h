@@ -97,8 +97,12 @@ struct GemmParams {
   int int1_direct = 1;
 };
 
-// Bytes of workspace with which the 1-bit GEMM of this size runs in one pass.
+// Bytes of workspace with which the 1-bit GEMM of this size runs in one pass
+// from an fp4 copy of its operands.
 size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k);
+// Bytes of both operands in the tiled 1-bit layout (what the pipeline packs the
+// caller's bytes into when the GEMM multiplies the packed words as they are).
+size_t gemm_int1_tiles_bytes(size_t batch, size_t m, size_t n, size_t k);
 
 // 1-bit GEMM whose operands p.x / p.y are one byte per sample, planar
 // [batch][2][rows][k] (the pipeline's input): expanded straight into the

@@ -542,15 +542,16 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
 
 bool gemm_int1_can_take_bytes(const GemmParams &p) {
   if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return false;
-  if (p.workspace_bytes < gemm_int1_workspace_bytes(p.batch, p.nx, p.ny, p.k)) return false;
+  const size_t need = p.int1_direct ? gemm_int1_tiles_bytes(p.batch, p.nx, p.ny, p.k)
+                                    : gemm_int1_workspace_bytes(p.batch, p.nx, p.ny, p.k);
+  if (p.workspace_bytes < need) return false;
   return p.batch <= 32767 && 16 * (size_t)p.x_tiles <= 65535 && 16 * (size_t)p.y_tiles <= 65535;
 }
 
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
   if (!gemm_int1_can_take_bytes(p)) return hipErrorInvalidValue;
   if (p.int1_direct) {
-    // pack into the tiled 1-bit layout (a quarter of the workspace) and multiply
-    // the packed words as they are
+    // pack into the tiled 1-bit layout and multiply the packed words as they are
     const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
     const size_t x_bytes = (size_t)p.batch * p.x_tiles * k1_tiles * kTileBytes;
     char *ws_x = static_cast<char *>(p.workspace), *ws_y = ws_x + x_bytes;
@@ -600,6 +601,11 @@ hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) 
 size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k) {
   if (k == 0 || k > kMaxMfmaK) return 0;
   return batch * (ceil_div(m, kTileRows) + ceil_div(n, kTileRows)) * ceil_div(k, 128) * kTileBytes;
+}
+
+size_t gemm_int1_tiles_bytes(size_t batch, size_t m, size_t n, size_t k) {
+  if (k == 0 || k > kMaxMfmaK) return 0;
+  return batch * (ceil_div(m, kTileRows) + ceil_div(n, kTileRows)) * ceil_div(k, 512) * kTileBytes;
 }
 
 hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream) {

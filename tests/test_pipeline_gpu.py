@@ -139,6 +139,30 @@ def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
+@pytest.mark.parametrize("mode", ["direct", "expand"])
+def test_pipeline_int1_unaligned_input(mode, monkeypatch):
+    # input buffers that start at an odd address: the kernels that read the bytes 16 at a
+    # time fall back to byte loads
+    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
+    if mode == "expand":
+        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
+    else:
+        monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
+    B, M, N, K = 2, 150, 140, 1056
+    rng = np.random.default_rng(5)
+    a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8)
+    d_a = to_device(np.concatenate([np.zeros(1, np.uint8), a_bits * 7]))
+    d_b = to_device(np.concatenate([np.zeros(3, np.uint8), b_bits * 255]))
+    d_c = to_device(np.zeros(B * 2 * M * N, dtype=np.int32))
+    p = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                    cc.Variant.opt)
+    p.Run(d_a.data_ptr() + 1, d_b.data_ptr() + 3, d_c.data_ptr())
+    torch.cuda.synchronize()
+    want = orc.gemm(pack_rows(a_bits, B, M, K), pack_rows(b_bits, B, N, K), M, N, K, orc.INT1, orc.INT32)
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+
+
 @functools.lru_cache(maxsize=1)
 def _grouped_int1_case(B, M, N, K):
     """Two sets of random 1-bit operands (one byte per sample) and the oracle's C for each."""
