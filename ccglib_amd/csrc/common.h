@@ -78,6 +78,10 @@ struct GemmParams {
   unsigned nx, ny;      // logical (un-padded) rows of X and Y
   unsigned k;           // logical K in samples
   unsigned k_tiles;     // number of 64-byte K tiles (ceil)
+  // When a launch covers only a piece of K (x and y then point at the piece's
+  // first tile or byte of row 0): K of the whole operand in memory, which sets
+  // the distance between rows and between row tiles. 0: the same as k.
+  unsigned k_in_memory = 0;
   unsigned x_tiles, y_tiles;  // 128-row tiles per operand (ceil)
   int type_in, type_out;
   int variant;          // kBasic: planar rows; kOpt: tiled layout

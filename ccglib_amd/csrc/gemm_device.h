@@ -94,6 +94,10 @@ struct KernelArgs {
   const char *y;
   char *c;
   unsigned batch, nx, ny, k, k_tiles, k_bytes, x_tiles, y_tiles;
+  // distance between consecutive rows of a planar operand (bytes) and between
+  // consecutive row tiles of a tiled one (K tiles): those of the whole operand
+  // in memory, of which this launch may cover a piece of K
+  unsigned row_stride_bytes, k_tile_stride;
   unsigned blocks_x, blocks_y;
   size_t x_batch_bytes, y_batch_bytes;
   float alpha_re, alpha_im, beta_re, beta_im;
@@ -156,14 +160,18 @@ inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
                                    : (unsigned)((size_t)p.k * bits_of(p.type_in) / 8);
   a.x_tiles = p.x_tiles;
   a.y_tiles = p.y_tiles;
+  const unsigned k_mem = p.k_in_memory ? p.k_in_memory : p.k;
+  a.row_stride_bytes = (p.type_in == kInt1) ? (unsigned)(ceil_div(k_mem, 32) * 4)
+                                            : (unsigned)((size_t)k_mem * bits_of(p.type_in) / 8);
+  a.k_tile_stride = p.k_in_memory ? (unsigned)ceil_div(k_mem, (size_t)k_per_tile(p.type_in)) : p.k_tiles;
   a.blocks_x = (unsigned)ceil_div(p.nx, bx);
   a.blocks_y = (unsigned)ceil_div(p.ny, by);
   if (p.variant == kOpt && !p.input_interleaved) {
-    a.x_batch_bytes = (size_t)p.x_tiles * p.k_tiles * kTileBytes;
-    a.y_batch_bytes = (size_t)p.y_tiles * p.k_tiles * kTileBytes;
+    a.x_batch_bytes = (size_t)p.x_tiles * a.k_tile_stride * kTileBytes;
+    a.y_batch_bytes = (size_t)p.y_tiles * a.k_tile_stride * kTileBytes;
   } else {
-    a.x_batch_bytes = (size_t)2 * p.nx * a.k_bytes;
-    a.y_batch_bytes = (size_t)2 * p.ny * a.k_bytes;
+    a.x_batch_bytes = (size_t)2 * p.nx * a.row_stride_bytes;
+    a.y_batch_bytes = (size_t)2 * p.ny * a.row_stride_bytes;
   }
   a.alpha_re = p.alpha_re;
   a.alpha_im = p.alpha_im;

@@ -486,7 +486,7 @@ hipError_t run_groups(const GemmParams &p, hipStream_t stream, size_t group, boo
 // the caller has checked), planar rows when they are whole aligned 16-byte
 // chunks (K a multiple of 128).
 bool direct_ok(const GemmParams &p) {
-  if (!p.int1_direct || p.k == 0 || p.k > kMaxMfmaK || p.input_interleaved) return false;
+  if (!p.int1_direct || p.k == 0 || p.input_interleaved) return false;
   if (((uintptr_t)p.x | (uintptr_t)p.y) % 16 != 0) return false;
   if (p.variant == kOpt) return true;
   const size_t k_bytes = ceil_div(p.k, 32) * 4;
@@ -497,7 +497,28 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
   *done = false;
   if (direct_ok(p)) {
     *done = true;
-    return launch_gemm_mfma(p, stream);
+    if (p.k <= kMaxMfmaK) return launch_gemm_mfma(p, stream);
+    // A longer K in pieces whose sums stay exact in fp32, each piece added to C
+    // by the integer epilogue: C = alpha S1 + beta C, then C += alpha S2, ...
+    // (whole tiles per piece; the operands' rows and row tiles keep the distances
+    // of the whole K)
+    const unsigned tiles_per_piece = kMaxMfmaK / 512;
+    for (unsigned t0 = 0; t0 < p.k_tiles; t0 += tiles_per_piece) {
+      GemmParams q = p;
+      q.k_in_memory = p.k;
+      q.k_tiles = std::min(tiles_per_piece, p.k_tiles - t0);
+      q.k = (t0 + q.k_tiles == p.k_tiles) ? p.k - t0 * 512 : q.k_tiles * 512;
+      const size_t offset = p.variant == kOpt ? (size_t)t0 * kTileBytes : (size_t)t0 * kTileRowBytes;
+      q.x = static_cast<const char *>(p.x) + offset;
+      q.y = static_cast<const char *>(p.y) + offset;
+      if (t0 > 0) {
+        q.beta_re = 1.f;
+        q.beta_im = 0.f;
+        q.have_beta = 1;
+      }
+      if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
+    }
+    return hipSuccess;
   }
   if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
   const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);

@@ -1389,6 +1389,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const unsigned total = args.blocks_x * args.blocks_y * args.batch;
   // bytes of one operand row in memory (planar: one plane's row)
   const unsigned row_bytes = IL ? 2 * args.k_bytes : args.k_bytes;
+  // ... and the distance between rows (larger when the launch covers a piece of K)
+  const unsigned row_stride = IL ? 2 * args.row_stride_bytes : args.row_stride_bytes;
 
   // ---- this wave's share of the copy: LPW row blocks of every K tile ------
   // Row block q of a slot: X re, X im, Y re, Y im, 16 rows each. What depends
@@ -1443,12 +1445,12 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
           unsigned tile = row0 / kTileRows;
           tile = tile < tiles ? tile : tiles - 1;   // rows past the end: never stored
-          src[i] = op + (size_t)tile * k_tiles * kTileBytes;
+          src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes;
         } else {
           const unsigned total_rows = is_x ? args.nx : args.ny;
           unsigned row = row0 + r;
           row = row < total_rows ? row : total_rows - 1;   // likewise
-          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_bytes + c_of(rb) * 16;
+          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_stride + c_of(rb) * 16;
         }
       }
     }

@@ -372,10 +372,10 @@ def test_int1_k_not_multiple_of_a_tile(K, int1_kernel):
     int1_case(2, 130, 70, K, cc.Variant.basic, seed=K + 2)
 
 
-def test_int1_largest_k_of_the_mfma_path_and_beyond():
-    # K = 2^22 is the largest the fp4 path takes (sums up to 2 K = 2^23 stay exact in
-    # fp32); identical operands give the extreme value im = 2 K in every element.
-    # One tile more and the popcount kernel takes over.
+def test_int1_largest_k_of_one_mfma_launch_and_beyond():
+    # K = 2^22 is the largest K of one launch on the fp4 MFMA (sums up to 2 K = 2^23 stay
+    # exact in fp32); identical operands give the extreme value im = 2 K in every element.
+    # A longer K is multiplied in pieces of 2^22 samples that the integer epilogue adds up.
     for K in (1 << 22, (1 << 22) + 512):
         kw = K // 32
         rng = np.random.default_rng(K)
@@ -389,6 +389,15 @@ def test_int1_largest_k_of_the_mfma_path_and_beyond():
         torch.cuda.synchronize()
         got = to_host(d_c, np.int32).reshape(2, 8, 4)
         assert (got[0] == 0).all() and (got[1] == 2 * K).all()
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+@pytest.mark.parametrize("K", [(1 << 22) + 128, 2 * (1 << 22) + 4096 + 96])
+def test_int1_k_in_pieces(variant, K, int1_kernel):
+    # two and three pieces, the last one a partial tile; alpha and beta applied once
+    if variant == cc.Variant.basic and K % 128:
+        K -= K % 128       # planar rows of whole 16-byte chunks, or the popcount kernel runs
+    int1_case(2, 40, 24, K, variant, c_order=COL, alpha=2 - 1j, beta=1 + 3j, seed=K % 1000)
 
 
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
