@@ -303,6 +303,9 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
   g->alpha_im = alpha_im;
   g->beta_re = beta_re;
   g->beta_im = beta_im;
+  const char *retile_env = std::getenv("CCGLIB_AMD_BASIC_RETILE");
+  const bool retile_allowed = !(retile_env && std::strcmp(retile_env, "0") == 0);
+  bool int1_retile = false;
   if (type_in == kInt1 && B && M && N) {
     // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs,
     // =expand on the MFMA kernel that reads an fp4 copy of the operands;
@@ -313,8 +316,13 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
     g->int1_direct = !(popcount || (kernel && std::strcmp(kernel, "expand") == 0));
     // The default kernel multiplies the packed words as they are and needs no
     // copy; only planar rows that are not whole 16-byte chunks go through one.
+    // Such rows are re-tiled first (below), unless CCGLIB_AMD_BASIC_RETILE=0, in
+    // which case the kernel on an fp4 copy multiplies them.
     const bool rows_direct = variant == kOpt || (ceil_div(K, 32) * 4) % 16 == 0;
-    size_t bytes = (g->int1_direct && rows_direct) ? 0 : gemm_int1_workspace_bytes(B, M, N, K);
+    int1_retile = g->int1_direct && !rows_direct && K > 0 && retile_allowed;
+    size_t bytes = (g->int1_direct && (rows_direct || int1_retile))
+                       ? 0
+                       : gemm_int1_workspace_bytes(B, M, N, K);
     const size_t per_batch = bytes / B;
     size_t cap = int1_workspace_cap();
     if (cap < per_batch) cap = per_batch;
@@ -342,18 +350,17 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
       }
     }
   }
-  const size_t eb = (size_t)bits_of(type_in) / 8;
-  const char *retile_env = std::getenv("CCGLIB_AMD_BASIC_RETILE");
-  if (type_in != kInt1 && variant == kBasic && B && M && N && K && (K * eb) % 16 != 0 &&
-      !(retile_env && std::strcmp(retile_env, "0") == 0)) {
+  const size_t bits = (size_t)bits_of(type_in);
+  if (variant == kBasic && B && M && N && K && retile_allowed &&
+      (type_in == kInt1 ? int1_retile : (K * bits / 8) % 16 != 0)) {
     // Rows that direct-to-LDS copies cannot fetch in whole chunks. Re-tiling them
     // costs two bandwidth-bound passes and a copy of A and B; the kernel for the
     // tiled layout then runs several times faster than the one that loads ragged
     // rows through registers. Without the memory that kernel is used.
     const size_t kc = (size_t)k_per_tile(type_in);
     const size_t kp = ceil_div(K, kc) * kc;
-    const size_t bytes_a = B * 2 * ceil_div(M, kTileRows) * kTileRows * kp * eb;
-    const size_t bytes_b = B * 2 * ceil_div(N, kTileRows) * kTileRows * kp * eb;
+    const size_t bytes_a = B * 2 * ceil_div(M, kTileRows) * kTileRows * kp * bits / 8;
+    const size_t bytes_b = B * 2 * ceil_div(N, kTileRows) * kTileRows * kp * bits / 8;
     DeviceGuard guard(device);
     if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes_a + bytes_b) == hipSuccess) {
       g->workspace_bytes = bytes_a + bytes_b;
@@ -392,10 +399,12 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   if (g->retile) {
     TransposeParams t;
     t.batch = g->B;
-    t.n = g->K;
+    // (1-bit rows are moved as 32-bit words)
+    const bool words = (g->type_in == kInt1);
+    t.n = words ? ceil_div(g->K, 32) : g->K;
     t.m_chunk = kTileRows;
-    t.n_chunk = (size_t)k_per_tile(g->type_in);
-    t.elem_bytes = bits_of(g->type_in) / 8;
+    t.n_chunk = words ? (size_t)k_per_tile(kInt1) / 32 : (size_t)k_per_tile(g->type_in);
+    t.elem_bytes = words ? 4 : bits_of(g->type_in) / 8;
     t.interleaved = 0;
     char *tiled_a = static_cast<char *>(g->workspace), *tiled_b = tiled_a + g->retile_b_offset;
     t.in = d_a;

@@ -392,6 +392,14 @@ def test_int1_largest_k_of_one_mfma_launch_and_beyond():
 
 
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+@pytest.mark.parametrize("K", [256, 1152])
+def test_int1_several_c_tiles_per_block(variant, K):
+    # 6 x 4 x 9 C tiles of 256 x 128 for at most 256 persistent blocks, with one and
+    # three K tiles per C tile (fewer than the copy's lead, and more)
+    int1_case(6, 1024, 1100, K, variant, seed=K)
+
+
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
 @pytest.mark.parametrize("K", [(1 << 22) + 128, 2 * (1 << 22) + 4096 + 96])
 def test_int1_k_in_pieces(variant, K, int1_kernel):
     # two and three pieces, the last one a partial tile; alpha and beta applied once
