@@ -356,8 +356,9 @@ def test_int1(variant, c_order, M, N, K, int1_kernel):
 
 
 @pytest.mark.parametrize("c_order", [ROW, COL])
-def test_int1_interleaved_output(c_order, int1_kernel):
-    int1_case(2, 100, 60, 512, cc.Variant.opt, INTERLEAVED, c_order)
+@pytest.mark.parametrize("K", [512, 160])
+def test_int1_interleaved_output(c_order, K, int1_kernel):
+    int1_case(2, 100, 60, K, cc.Variant.opt, INTERLEAVED, c_order)
 
 
 @pytest.mark.parametrize("K", [45, 100, 1000])
