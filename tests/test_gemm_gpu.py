@@ -392,6 +392,25 @@ def test_int1_largest_k_of_one_mfma_launch_and_beyond():
         assert (got[0] == 0).all() and (got[1] == 2 * K).all()
 
 
+@pytest.mark.parametrize("K", [256, 96])
+def test_int1_basic_word_aligned_pointers(K, int1_kernel):
+    # planar rows that start at a word but not at a 16-byte boundary: no kernel may read
+    # them in 16-byte pieces
+    B, M, N = 2, 70, 90
+    rng = np.random.default_rng(K)
+    kw = K // 32
+    a = rng.integers(0, 2 ** 32, B * 2 * M * kw, dtype=np.uint32)
+    b = rng.integers(0, 2 ** 32, B * 2 * N * kw, dtype=np.uint32)
+    d_a = to_device(np.concatenate([np.zeros(1, np.uint32), a]))
+    d_b = to_device(np.concatenate([np.zeros(3, np.uint32), b]))
+    d_c = to_device(np.zeros(B * 2 * M * N, np.int32))
+    cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.int1, VT.int32), cc.Variant.basic).Run(
+        d_a.data_ptr() + 4, d_b.data_ptr() + 12, d_c.data_ptr())
+    torch.cuda.synchronize()
+    want = orc.gemm(a, b, M, N, K, orc.INT1, orc.INT32)
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+
+
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
 @pytest.mark.parametrize("K", [256, 1152])
 def test_int1_several_c_tiles_per_block(variant, K):
