@@ -1,10 +1,18 @@
-// 1-bit complex GEMM: XOR + population count on the vector ALU.
+// 1-bit complex GEMM.
 //
 // Stands in for the reference's int1 wmma_complex_gemm_basic / _opt
 // (kernels/gemm_kernel_int1.cu:64-196, :198-356), which exist for NVIDIA's
-// binary tensor-core op only; gfx950 has no 1-bit matrix instruction, so the
-// dot products are built from v_xor_b32 and v_bcnt_u32_b32 (whose add operand
-// does the accumulation). With bit 1 = +1 and bit 0 = -1 a product is an XOR
+// binary tensor-core op only; gfx950 has no 1-bit matrix instruction. This file
+// holds the launcher, which picks one of three ways to the same integers:
+//  * the fp4 MFMA kernel on the packed words as they are (in the file of the MFMA
+//    kernels; tiled operands and planar rows of whole 16-byte chunks),
+//  * the same MFMA on a copy of the operands expanded to fp4 (expand_* below),
+//  * XOR + population count on the vector ALU (complex_gemm_int1 below),
+// and the kernel that packs one byte per sample straight into 1-bit tiles for
+// the pipeline.
+//
+// The popcount kernel builds the dot products from v_xor_b32 and
+// v_bcnt_u32_b32 (whose add operand does the accumulation). With bit 1 = +1 and bit 0 = -1 a product is an XOR
 // and a sum a popcount (src/reference/GEMM.cpp:131-200):
 //   pop_re = popc(xr ^ yr) + popc(xi ^ ~yi)
 //   pop_im = popc(xr ^ yi) + popc(xi ^ yr)

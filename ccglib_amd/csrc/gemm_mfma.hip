@@ -1,5 +1,6 @@
-// Complex GEMM on the gfx950 matrix cores for fp16, bf16 and fp8 (e4m3/e5m2)
-// input with fp32 accumulation.
+// Complex GEMM on the gfx950 matrix cores for fp16, bf16, fp32 and fp8
+// (e4m3/e5m2) input with fp32 accumulation, and for 1-bit input (+-1 values on
+// the fp4 instruction, exact integer sums; kernels/gemm_kernel_int1.cu:64-356).
 //
 // Stands in for the reference's wmma_complex_gemm_basic / wmma_complex_gemm_opt
 // (kernels/gemm_kernel_float.cu:35-181, :186-355) and its epilogue helpers
