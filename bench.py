@@ -126,41 +126,11 @@ def check_result(name, a, b, c, torch):
             "batch": bi}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    # The part runs under a power limit whose controller takes about 30 ms of continuous
-    # load to settle (GEMM launches of the default workload go 0.55 -> 0.70 -> 0.56 ms over
-    # the first 35 steps): the default warm-up covers that, and the timed steps are the
-    # settled rate.
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="beamformer", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-check", action="store_true")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also launch a plain 1 GiB device copy (for scaling rocprofv3 HBM counters)")
-    ap.add_argument("--isolated", action="store_true",
-                    help="also time the GEMM launched back to back outside the step")
-    ap.add_argument("--host", action="store_true",
-                    help="also time Pipeline's host-pointer Run on page-locked buffers (copies over "
-                         "PCIe in both directions included; never part of `value`)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the batch axis "
-                 "would shard with no exchange); run with --gpus 1")
-
-    import numpy as np
-    import torch
-    import ccglib_amd as cc
-
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU")
-    torch.cuda.set_device(0)
+def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_calibration=False):
+    """Builds the step of a workload, settles, times `steps` steps and checks the result.
+    Returns a dict of figures plus what the optional extra measurements need."""
     stream = torch.cuda.current_stream().cuda_stream
     VT, AX, MO = cc.ValueType, cc.ComplexAxisLocation, cc.MemOrder
-
-    name = args.workload
     B, M, N, K, tin_name, tout_name, axis_name, description = WORKLOADS[name]
     tin, tout = VT[tin_name], VT[tout_name]
     axis = AX.complex_interleaved if axis_name == "interleaved" else AX.complex_planar
@@ -204,11 +174,26 @@ def main():
             fn()
         run_gemm()
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    # Settle phase, sized by duration as the reference's benchmark protocol sizes its warm-up
+    # (benchmark/benchmark_gemm.cpp:262-298): the part runs under a power limit whose
+    # controller needs tens of milliseconds of continuous load to reach its steady clock,
+    # whatever --warmup says. The same step, untimed, until `settle_ms` have passed.
+    settle_steps, settled = 0, 0.0
+    if settle_ms > 0:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        while settled < settle_ms:
+            e0.record()
+            for _ in range(8):
+                step()
+            e1.record()
+            e1.synchronize()
+            settled += e0.elapsed_time(e1)
+            settle_steps += 8
 
-    if args.copy_calibration:
+    if copy_calibration:
         # a copy kernel of known size: reads 1 GiB and writes 1 GiB per launch
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
         dst = torch.empty_like(src)
@@ -222,9 +207,10 @@ def main():
     # stream the kernels are launched on, which gives each kernel's duration in
     # the situation that counts (the GEMM right after the data preparation).
     nk = len(kernels)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(nk + 2)] for _ in range(args.steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(nk + 2)] for _ in range(steps)]
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         ev[i][0].record()
         for j, (_, fn, _) in enumerate(kernels):
             fn()
@@ -232,50 +218,35 @@ def main():
         run_gemm()
         ev[i][nk + 1].record()
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
 
     flops = 8.0 * B * M * N * K
-    value = flops / (ms_per_step * 1e-3) / 1e12
-    gemm_ms = sum(e[nk].elapsed_time(e[nk + 1]) for e in ev) / args.steps
+    gemm_ms = sum(e[nk].elapsed_time(e[nk + 1]) for e in ev) / steps
     gemm_tflops = flops / (gemm_ms * 1e-3) / 1e12
     per_kernel = {"gemm_ms": gemm_ms, "gemm_tflops": gemm_tflops}
     for j, (label, _, nbytes) in enumerate(kernels):
-        ms = sum(e[j].elapsed_time(e[j + 1]) for e in ev) / args.steps
+        ms = sum(e[j].elapsed_time(e[j + 1]) for e in ev) / steps
         per_kernel[label + "_ms"] = ms
         per_kernel[label + "_gbs"] = nbytes / ms / 1e6
         per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
 
     if tin == VT.int1:
-        dtype, peak, bound, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "mfma", "TOP/s"
+        dtype, peak, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "TOP/s"
         kernel_name = "complex_gemm_mfma_dtl<int1->int32> (fp4 MFMA, bits expanded in registers)"
     else:
         dtype = {"float16": "f16", "bfloat16": "bf16"}.get(tin_name, "fp8")
-        peak, bound, unit = MFMA_PEAK_TFLOPS[dtype], "mfma", "TFLOP/s"
+        peak, unit = MFMA_PEAK_TFLOPS[dtype], "TFLOP/s"
         kernel_name = "complex_gemm_mfma_dtl<%s->%s>" % (tin_name, tout_name)
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemm_f16_beamformer_traffic.json")
-    if name == "beamformer" and os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-
-    result = {
-        "metric": "complex TFLOP/s (8 flop/cMAC) on 1 MI355X + % of dtype MFMA peak",
-        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": description + " (data preparation kernels inside the step)",
-                   "name": name, "B": B, "M": M, "N": N, "K": K, "variant": "opt"},
-        "pct_of_peak": 100.0 * value / peak,
-        "roofline": {"kernel": kernel_name, "bound": bound, "achieved": gemm_tflops, "peak": peak,
-                     "unit": unit, "frac": gemm_tflops / peak, "traffic": traffic,
-                     "kernel_ms": gemm_ms},
-        "kernels": per_kernel,
-    }
-    result.update(info)
-
-    if args.isolated:
+    out = {"name": name, "description": description, "shape": (B, M, N, K), "flops": flops,
+           "ms_per_step": ms_per_step, "value": flops / (ms_per_step * 1e-3) / 1e12,
+           "gemm_ms": gemm_ms, "gemm_tflops": gemm_tflops, "per_kernel": per_kernel,
+           "dtype": dtype, "peak": peak, "unit": unit, "kernel_name": kernel_name,
+           "settle_ms": settled, "settle_steps": settle_steps, "info": info,
+           "check": check_result(name, a_in, b_in, c, torch)}
+    if isolated:
         # the GEMM launched back to back on its own (inputs and caches warm)
-        iters = max(args.steps, 10)
+        iters = max(steps, 10)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         run_gemm()
         torch.cuda.synchronize()
@@ -285,8 +256,83 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         iso_ms = e0.elapsed_time(e1) / iters
-        result["isolated"] = {"gemm_ms": iso_ms, "gemm_tflops": flops / (iso_ms * 1e-3) / 1e12}
+        out["isolated"] = {"gemm_ms": iso_ms, "gemm_tflops": flops / (iso_ms * 1e-3) / 1e12}
+    out["_buffers"] = (a_in, b_in, c)    # for the optional pipeline measurements of the caller
+    return out
 
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    # The part runs under a power limit whose controller takes about 30 ms of continuous
+    # load to settle (GEMM launches of the default workload go 0.55 -> 0.70 -> 0.56 ms over
+    # the first 35 steps). Whatever --warmup says, the same step is repeated, untimed, for
+    # this many milliseconds before the timed region, and the JSON line says so.
+    ap.add_argument("--settle-ms", type=float, default=150.0)
+    ap.add_argument("--workload", default="beamformer", choices=sorted(WORKLOADS))
+    ap.add_argument("--other-steps", type=int, default=20,
+                    help="timed steps of each of the other workloads that a default run reports "
+                         "in `other_workloads` (0: skip them)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 1 GiB device copy (for scaling rocprofv3 HBM counters)")
+    ap.add_argument("--isolated", action="store_true",
+                    help="also time the GEMM launched back to back outside the step")
+    ap.add_argument("--host", action="store_true",
+                    help="also time Pipeline's host-pointer Run on page-locked buffers (copies over "
+                         "PCIe in both directions included; never part of `value`)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the batch axis "
+                 "would shard with no exchange); run with --gpus 1")
+
+    import numpy as np
+    import torch
+    import ccglib_amd as cc
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    VT, AX, MO = cc.ValueType, cc.ComplexAxisLocation, cc.MemOrder
+
+    name = args.workload
+    B, M, N, K, tin_name, tout_name, axis_name, description = WORKLOADS[name]
+    tin, tout = VT[tin_name], VT[tout_name]
+    m = measure(name, args.steps, args.warmup, args.settle_ms, torch, np, cc,
+                isolated=args.isolated, copy_calibration=args.copy_calibration)
+    a_in, b_in, c = m.pop("_buffers")
+    flops, value, ms_per_step = m["flops"], m["value"], m["ms_per_step"]
+    gemm_ms, gemm_tflops, peak = m["gemm_ms"], m["gemm_tflops"], m["peak"]
+
+    traffic, traffic_source = None, None
+    tpath = os.path.join(ROOT, "profiles", "gemm_f16_beamformer_traffic.json")
+    if name == "beamformer" and os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        traffic_source = ("constant read from profiles/gemm_f16_beamformer_traffic.json: rocprofv3 "
+                          "--pmc FETCH_SIZE / WRITE_SIZE of this command in an earlier run, scaled "
+                          "by a copy kernel; not measured in this run")
+
+    result = {
+        "metric": "complex TFLOP/s (8 flop/cMAC) on 1 MI355X + % of dtype MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "settle_ms": m["settle_ms"], "settle_steps": m["settle_steps"],
+        "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": m["dtype"], "data": "synthetic",
+        "config": {"workload": description + " (data preparation kernels inside the step)",
+                   "name": name, "B": B, "M": M, "N": N, "K": K, "variant": "opt"},
+        "pct_of_peak": 100.0 * value / peak,
+        "roofline": {"kernel": m["kernel_name"], "bound": "mfma", "achieved": gemm_tflops,
+                     "peak": peak, "unit": m["unit"], "frac": gemm_tflops / peak,
+                     "traffic": traffic, "traffic_source": traffic_source, "kernel_ms": gemm_ms},
+        "kernels": m["per_kernel"],
+    }
+    result.update(m["info"])
+    if "isolated" in m:
+        result["isolated"] = m["isolated"]
 
     if axis_name == "interleaved":
         # The same job through ccglib's Pipeline wrapper, which here feeds the interleaved
@@ -295,7 +341,7 @@ def main():
         c2 = torch.empty_like(c)
         pipe = cc.Pipeline(B, M, N, K, 0, stream, AX.complex_interleaved, AX.complex_planar,
                            MO.row_major, MO.col_major, MO.row_major, tin, tout, cc.Variant.opt)
-        for _ in range(args.warmup):
+        for _ in range(args.warmup + m["settle_steps"]):
             pipe.Run(a_in.data_ptr(), b_in.data_ptr(), c2.data_ptr())
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -313,7 +359,7 @@ def main():
         c2 = torch.empty_like(c)
         pipe = cc.Pipeline(B, M, N, K, 0, stream, AX.complex_planar, AX.complex_planar,
                            MO.row_major, MO.col_major, MO.row_major, tin, tout, cc.Variant.opt)
-        for _ in range(args.warmup):
+        for _ in range(args.warmup + m["settle_steps"]):
             pipe.Run(a_in.data_ptr(), b_in.data_ptr(), c2.data_ptr())
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -358,7 +404,28 @@ def main():
         del pipe, h_a, h_b, h_c
 
     if not args.no_check:
-        result["check"] = check_result(name, a_in, b_in, c, torch)
+        result["check"] = m["check"]
+
+    if name == "beamformer" and args.other_steps > 0:
+        # The reference's other benchmark configurations under the same clock: the same
+        # protocol (warm-up, settle phase, events around the GEMM inside the step), fewer
+        # steps; the buffers of one workload are freed before the next one is built.
+        del a_in, b_in, c, m
+        torch.cuda.empty_cache()
+        others = {}
+        for other in ("square_bf16", "fp8_e4m3", "correlator_int1"):
+            o = measure(other, args.other_steps, 3, args.settle_ms, torch, np, cc)
+            o.pop("_buffers")
+            others[other] = {
+                "kernel": o["kernel_name"], "shape": dict(zip("BMNK", o["shape"])),
+                "steps": args.other_steps, "settle_ms": o["settle_ms"],
+                "kernel_ms": o["gemm_ms"], "achieved": o["gemm_tflops"], "peak": o["peak"],
+                "unit": o["unit"], "frac": o["gemm_tflops"] / o["peak"],
+                "ms_per_step": o["ms_per_step"], "step_rate": o["value"],
+                "kernels": o["per_kernel"], "check": o["check"]}
+            del o
+            torch.cuda.empty_cache()
+        result["other_workloads"] = others
 
     if not args.no_cpu_baseline and name == "beamformer":
         import oracle as orc

@@ -13,6 +13,7 @@ streams as integer ``hipStream_t`` handles (0 = default stream). Every ``Run``
 only enqueues work on the stream. Errors raise ``RuntimeError`` with the
 library's message, as the reference throws ``std::runtime_error``.
 """
+import contextlib
 import ctypes
 import enum
 
@@ -83,6 +84,35 @@ def ceildiv(a, b):
 
 def version():
     return _capi.load().ccglib_version().decode()
+
+
+class Option(enum.IntEnum):
+    """Process-wide options of the library (include/ccglib_amd.h; no counterpart in
+    the reference). Read when an object is created."""
+    int1_popcount = 0
+    basic_retile = 1
+    host_chunk_bytes = 2
+
+
+def set_option(option, value):
+    _capi.check(_capi.load().ccglib_amd_set_option(int(option), int(value)))
+
+
+def get_option(option):
+    out = ctypes.c_size_t(0)
+    _capi.check(_capi.load().ccglib_amd_get_option(int(option), ctypes.byref(out)))
+    return out.value
+
+
+@contextlib.contextmanager
+def option(option, value):
+    """Sets an option for the duration of a with block."""
+    old = get_option(option)
+    set_option(option, value)
+    try:
+        yield
+    finally:
+        set_option(option, old)
 
 
 def _ptr(x):
@@ -192,3 +222,4 @@ class Pipeline(_Handle):
     def RunHost(self, h_a, h_b, h_c):
         _capi.check(_capi.load().ccglib_pipeline_run_host(self._h, _ptr(h_a), _ptr(h_b),
                                                          _ptr(h_c)))
+

@@ -4,6 +4,7 @@
 // src/transpose/Transpose.cpp, src/packing/Packing.cpp,
 // src/pipeline/Pipeline.cpp.
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -103,19 +104,20 @@ struct ccglib_gemm {
   // Set by the pipeline only: A and B are the caller's interleaved (re, im)
   // rows and are consumed as they are, without a transpose.
   bool input_interleaved = false;
-  // 1-bit GEMM: device memory for the operands expanded for the MFMA path
-  // (null: the popcount kernel runs instead)
+  // Device memory the object owns (freed with it): the tiled copies of a
+  // basic-variant GEMM (below), or, for the 1-bit pipeline, the 1-bit tiles
+  // that the caller's bytes are packed into.
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
-  // 1-bit GEMM with a workspace: a second stream on which the expansion of later
-  // batches runs while earlier ones are multiplied (null members: not in use)
-  GemmAux aux;
-  // Basic variant with rows that are not whole 16-byte chunks (odd K): A and B
-  // are first copied into the tiled layout (A at the start of `workspace`, B at
-  // retile_b_offset) and the kernel of the opt variant runs on the copies.
-  bool retile = false;
+  // Basic variant whose planar rows direct-to-LDS copies cannot fetch (rows that
+  // are not whole 16-byte chunks, or operands that are not 16-byte aligned): A
+  // and B are first copied into the tiled layout (A at the start of
+  // `workspace`, B at retile_b_offset) and the kernel of the opt variant runs on
+  // the copies. retile_allowed: the option was on when the object was created.
+  bool retile = false, retile_allowed = true;
   size_t retile_b_offset = 0;
-  // 1-bit GEMM: the MFMA kernel may read the packed words as they are
+  // 1-bit GEMM: the MFMA kernel multiplies the packed words (0: the option that
+  // keeps it on the vector ALUs was set when the object was created)
   int int1_direct = 1;
 };
 
@@ -131,6 +133,9 @@ struct ccglib_packing {
   size_t N;
   int direction, device, axis;
   hipStream_t stream;
+  // Set by the pipeline only: interleaved input is this many buffers of
+  // N / segments samples, one after the other, each packed on its own.
+  size_t segments = 1;
 };
 
 struct ccglib_pipeline {
@@ -142,6 +147,11 @@ struct ccglib_pipeline {
   // 1-bit input, one byte per sample, planar: expanded straight into the GEMM's
   // workspace (no packed or transposed intermediates)
   bool int1_direct = false;
+  // 8/16-bit interleaved input that the GEMM reads in place (no transposes);
+  // `unfused` is the pipeline with transposes that takes over for buffers that
+  // are not 16-byte aligned, created by the first Run that meets such buffers
+  bool fused = false;
+  ccglib_pipeline *unfused = nullptr;
   ccglib_packing_t pack_a = nullptr, pack_b = nullptr;
   ccglib_transpose_t trans_a = nullptr, trans_b = nullptr;
   ccglib_gemm_t gemm = nullptr;
@@ -166,21 +176,38 @@ struct ccglib_pipeline {
 
 namespace {
 
-void release_aux(GemmAux *aux) {
-  for (int i = 0; i < GemmAux::kMaxJoins; ++i) {
-    if (aux->join[i]) (void)hipEventDestroy(aux->join[i]);
-    aux->join[i] = nullptr;
-  }
-  if (aux->fork) (void)hipEventDestroy(aux->fork);
-  if (aux->stream) (void)hipStreamDestroy(aux->stream);
-  aux->fork = nullptr;
-  aux->stream = nullptr;
+// Process-wide options (ccglib_amd_set_option), read when an object is created.
+size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0};
+
+// Largest buffer of 1-bit tiles a pipeline allocates; beyond it the pipeline
+// runs the reference's sequence of kernels on its packed / transposed buffers.
+constexpr size_t kInt1TilesCap = (size_t)16 << 30;
+
+// Bytes of A and of B in the tiled layout (whole tiles).
+void tiled_bytes(const ccglib_gemm *g, size_t *bytes_a, size_t *bytes_b) {
+  const size_t bits = (size_t)bits_of(g->type_in);
+  const size_t kc = (size_t)k_per_tile(g->type_in);
+  const size_t kp = ceil_div(g->K, kc) * kc;
+  *bytes_a = g->B * 2 * ceil_div(g->M, kTileRows) * kTileRows * kp * bits / 8;
+  *bytes_b = g->B * 2 * ceil_div(g->N, kTileRows) * kTileRows * kp * bits / 8;
 }
 
-// Largest workspace a 1-bit GEMM object allocates (CCGLIB_AMD_INT1_WORKSPACE_MB, default 16 GiB).
-size_t int1_workspace_cap() {
-  const char *cap_mb = std::getenv("CCGLIB_AMD_INT1_WORKSPACE_MB");
-  return cap_mb ? (size_t)std::strtoull(cap_mb, nullptr, 10) << 20 : (size_t)16 << 30;
+// Gives a basic-variant GEMM the workspace for tiled copies of its operands.
+// Failing to get the memory is not an error: the kernels that read planar rows
+// in place then run.
+void make_retile_workspace(ccglib_gemm *g) {
+  if (g->workspace || !g->retile_allowed) return;
+  size_t bytes_a = 0, bytes_b = 0;
+  tiled_bytes(g, &bytes_a, &bytes_b);
+  DeviceGuard guard(g->device);
+  if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes_a + bytes_b) == hipSuccess) {
+    g->workspace_bytes = bytes_a + bytes_b;
+    g->retile = true;
+    g->retile_b_offset = bytes_a;
+  } else {
+    g->workspace = nullptr;
+    (void)hipGetLastError();
+  }
 }
 
 // Launch parameters of a GEMM object for the given buffers.
@@ -221,8 +248,69 @@ void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, vo
   p.have_beta = (g->beta_re != 0.0f || g->beta_im != 0.0f);
   p.workspace = g->workspace;
   p.workspace_bytes = g->workspace_bytes;
-  p.aux = g->aux.stream ? &g->aux : nullptr;
   p.int1_direct = g->int1_direct;
+}
+
+}  // namespace
+
+namespace {
+
+// Argument checks shared by the GEMM constructor and the stateless entry point,
+// in the reference's order and with its wording.
+int validate_gemm(size_t B, size_t M, size_t N, size_t K, int type_in, int type_out, int variant,
+                  int c_complex_axis_location, int c_mem_order, int a_mem_order, int b_mem_order) {
+  if (!is_enum01(variant) || !is_enum01(c_complex_axis_location) || !is_enum01(c_mem_order) ||
+      !is_enum01(a_mem_order) || !is_enum01(b_mem_order)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  if (variant == kBasic && c_complex_axis_location == kInterleaved) {
+    // src/mma/GEMM.cpp:77-80
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "complex-interleaved output is not supported in basic variant");
+  }
+  if (!pair_supported(type_in, type_out)) {
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "No kernel parameters available for selected precision (in %d, out %d)", type_in,
+                type_out);
+  }
+  if (a_mem_order != kRowMajor || b_mem_order != kColMajor) {
+    // The reference rejects these layouts when it compiles its kernel at
+    // construction (kernels/gemm_kernel_float.cu:20-25); callers match on the
+    // name of that failure (test/gemm/mma.cpp:598-627).
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "HIPRTC_ERROR_COMPILATION: GEMM supports only a row-major A matrix and a "
+                "col-major B matrix");
+  }
+  if (B > 0xffffffffu || M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "problem size out of range");
+  }
+  // the kernels address a row with 32-bit byte offsets, also when the pipeline
+  // hands them interleaved rows (twice the bytes)
+  if (2 * K * (size_t)bits_of(type_in) / 8 > 0xffffffffu) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                "K = %zu: a row of the operands must stay below 2 GiB", K);
+  }
+  return CCGLIB_OK;
+}
+
+void init_gemm(ccglib_gemm *g, size_t B, size_t M, size_t N, size_t K, int device, void *stream,
+               int type_in, int type_out, int variant, int c_complex_axis_location,
+               int c_mem_order, float alpha_re, float alpha_im, float beta_re, float beta_im) {
+  g->B = B;
+  g->M = M;
+  g->N = N;
+  g->K = K;
+  g->device = device;
+  g->stream = static_cast<hipStream_t>(stream);
+  g->type_in = type_in;
+  g->type_out = type_out;
+  g->variant = variant;
+  g->c_axis = c_complex_axis_location;
+  g->c_order = c_mem_order;
+  g->alpha_re = alpha_re;
+  g->alpha_im = alpha_im;
+  g->beta_re = beta_re;
+  g->beta_im = beta_im;
 }
 
 }  // namespace
@@ -231,7 +319,23 @@ extern "C" {
 
 const char *ccglib_last_error(void) { return g_last_error.c_str(); }
 
-const char *ccglib_version(void) { return "ccglib-amd 0.1.0 (gfx950)"; }
+const char *ccglib_version(void) { return "ccglib-amd 0.2.0 (gfx950)"; }
+
+int ccglib_amd_set_option(int option, size_t value) {
+  if (option < 0 || option >= CCGLIB_AMD_OPTION_COUNT) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "unknown option %d", option);
+  }
+  g_options[option] = value;
+  return CCGLIB_OK;
+}
+
+int ccglib_amd_get_option(int option, size_t *value) {
+  if (option < 0 || option >= CCGLIB_AMD_OPTION_COUNT || !value) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "unknown option %d", option);
+  }
+  *value = g_options[option];
+  return CCGLIB_OK;
+}
 
 /* ------------------------------- GEMM ---------------------------------- */
 
@@ -260,116 +364,26 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
                        float beta_im) {
   if (!gemm) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
   *gemm = nullptr;
-  if (!is_enum01(variant) || !is_enum01(c_complex_axis_location) || !is_enum01(c_mem_order) ||
-      !is_enum01(a_mem_order) || !is_enum01(b_mem_order)) {
-    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
-  }
-  if (variant == kBasic && c_complex_axis_location == kInterleaved) {
-    // src/mma/GEMM.cpp:77-80
-    return fail(CCGLIB_ERROR_UNSUPPORTED,
-                "complex-interleaved output is not supported in basic variant");
-  }
-  if (!pair_supported(type_in, type_out)) {
-    return fail(CCGLIB_ERROR_UNSUPPORTED,
-                "No kernel parameters available for selected precision (in %d, out %d)", type_in,
-                type_out);
-  }
-  if (a_mem_order != kRowMajor || b_mem_order != kColMajor) {
-    // The reference rejects these layouts when it compiles its kernel at
-    // construction (kernels/gemm_kernel_float.cu:20-25); callers match on the
-    // name of that failure (test/gemm/mma.cpp:598-627).
-    return fail(CCGLIB_ERROR_UNSUPPORTED,
-                "HIPRTC_ERROR_COMPILATION: GEMM supports only a row-major A matrix and a "
-                "col-major B matrix");
-  }
-  if (B > 0xffffffffu || M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu) {
-    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "problem size out of range");
+  if (int rc = validate_gemm(B, M, N, K, type_in, type_out, variant, c_complex_axis_location,
+                             c_mem_order, a_mem_order, b_mem_order)) {
+    return rc;
   }
   if (int rc = check_device(device)) return rc;
   ccglib_gemm *g = new (std::nothrow) ccglib_gemm;
   if (!g) return fail(CCGLIB_ERROR_RUNTIME, "out of host memory");
-  g->B = B;
-  g->M = M;
-  g->N = N;
-  g->K = K;
-  g->device = device;
-  g->stream = static_cast<hipStream_t>(stream);
-  g->type_in = type_in;
-  g->type_out = type_out;
-  g->variant = variant;
-  g->c_axis = c_complex_axis_location;
-  g->c_order = c_mem_order;
-  g->alpha_re = alpha_re;
-  g->alpha_im = alpha_im;
-  g->beta_re = beta_re;
-  g->beta_im = beta_im;
-  const char *retile_env = std::getenv("CCGLIB_AMD_BASIC_RETILE");
-  const bool retile_allowed = !(retile_env && std::strcmp(retile_env, "0") == 0);
-  bool int1_retile = false;
-  if (type_in == kInt1 && B && M && N) {
-    // CCGLIB_AMD_INT1_KERNEL=popcount keeps the 1-bit GEMM on the vector ALUs,
-    // =expand on the MFMA kernel that reads an fp4 copy of the operands;
-    // CCGLIB_AMD_INT1_WORKSPACE_MB caps that copy (the GEMM then runs in groups
-    // of batches). Failing to get the memory is not an error.
-    const char *kernel = std::getenv("CCGLIB_AMD_INT1_KERNEL");
-    const bool popcount = kernel && std::strcmp(kernel, "popcount") == 0;
-    g->int1_direct = !(popcount || (kernel && std::strcmp(kernel, "expand") == 0));
-    // The default kernel multiplies the packed words as they are and needs no
-    // copy; only planar rows that are not whole 16-byte chunks go through one.
-    // Such rows are re-tiled first (below), unless CCGLIB_AMD_BASIC_RETILE=0, in
-    // which case the kernel on an fp4 copy multiplies them.
-    const bool rows_direct = variant == kOpt || (ceil_div(K, 32) * 4) % 16 == 0;
-    int1_retile = g->int1_direct && !rows_direct && K > 0 && retile_allowed;
-    size_t bytes = (g->int1_direct && (rows_direct || int1_retile))
-                       ? 0
-                       : gemm_int1_workspace_bytes(B, M, N, K);
-    const size_t per_batch = bytes / B;
-    size_t cap = int1_workspace_cap();
-    if (cap < per_batch) cap = per_batch;
-    if (bytes > cap) bytes = cap / per_batch * per_batch;
-    if (bytes && !popcount) {
-      DeviceGuard guard(device);
-      if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes) == hipSuccess) {
-        g->workspace_bytes = bytes;
-        // CCGLIB_AMD_INT1_OVERLAP=0 keeps everything on the caller's stream
-        const char *overlap = std::getenv("CCGLIB_AMD_INT1_OVERLAP");
-        if (!(overlap && std::strcmp(overlap, "0") == 0)) {
-          hipError_t e = hipStreamCreateWithFlags(&g->aux.stream, hipStreamNonBlocking);
-          if (e == hipSuccess) e = hipEventCreateWithFlags(&g->aux.fork, hipEventDisableTiming);
-          for (int i = 0; i < GemmAux::kMaxJoins && e == hipSuccess; ++i) {
-            e = hipEventCreateWithFlags(&g->aux.join[i], hipEventDisableTiming);
-          }
-          if (e != hipSuccess) {   // not an error: the GEMM then runs on one stream
-            release_aux(&g->aux);
-            (void)hipGetLastError();
-          }
-        }
-      } else {
-        g->workspace = nullptr;
-        (void)hipGetLastError();
-      }
-    }
-  }
-  const size_t bits = (size_t)bits_of(type_in);
-  if (variant == kBasic && B && M && N && K && retile_allowed &&
-      (type_in == kInt1 ? int1_retile : (K * bits / 8) % 16 != 0)) {
-    // Rows that direct-to-LDS copies cannot fetch in whole chunks. Re-tiling them
-    // costs two bandwidth-bound passes and a copy of A and B; the kernel for the
-    // tiled layout then runs several times faster than the one that loads ragged
-    // rows through registers. Without the memory that kernel is used.
-    const size_t kc = (size_t)k_per_tile(type_in);
-    const size_t kp = ceil_div(K, kc) * kc;
-    const size_t bytes_a = B * 2 * ceil_div(M, kTileRows) * kTileRows * kp * bits / 8;
-    const size_t bytes_b = B * 2 * ceil_div(N, kTileRows) * kTileRows * kp * bits / 8;
-    DeviceGuard guard(device);
-    if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes_a + bytes_b) == hipSuccess) {
-      g->workspace_bytes = bytes_a + bytes_b;
-      g->retile = true;
-      g->retile_b_offset = bytes_a;
-    } else {
-      g->workspace = nullptr;
-      (void)hipGetLastError();
-    }
+  init_gemm(g, B, M, N, K, device, stream, type_in, type_out, variant, c_complex_axis_location,
+            c_mem_order, alpha_re, alpha_im, beta_re, beta_im);
+  g->retile_allowed = g_options[CCGLIB_AMD_OPTION_BASIC_RETILE] != 0;
+  g->int1_direct = g_options[CCGLIB_AMD_OPTION_INT1_POPCOUNT] == 0;
+  // Planar rows that direct-to-LDS copies cannot fetch in whole chunks (for 1-bit
+  // input: rows of K / 32 words). Re-tiling them costs two bandwidth-bound passes
+  // and a copy of A and B; the kernel for the tiled layout then runs several
+  // times faster than the ones that load ragged rows through registers.
+  // (Operands that are not 16-byte aligned get the same workspace at their first Run.)
+  const size_t row_bytes = type_in == kInt1 ? ceil_div(K, 32) * 4 : K * (size_t)bits_of(type_in) / 8;
+  if (variant == kBasic && B && M && N && K && row_bytes % 16 != 0 &&
+      (type_in != kInt1 || g->int1_direct)) {
+    make_retile_workspace(g);
   }
   *gemm = g;
   return CCGLIB_OK;
@@ -396,7 +410,18 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   }
   DeviceGuard guard(g->device);
   HIP_TRY(guard.status());
-  if (g->retile) {
+  bool retile_now = g->retile;
+  if (g->variant == kBasic && g->K && (g->type_in != kInt1 || g->int1_direct)) {
+    const size_t row_bytes = g->type_in == kInt1 ? ceil_div(g->K, 32) * 4
+                                                 : g->K * (size_t)bits_of(g->type_in) / 8;
+    const bool misaligned = (uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0;
+    // Planar operands that are not 16-byte aligned cannot be copied to LDS in
+    // place either: the object gets its workspace at the first such Run (the one
+    // allocation a Run may make) and keeps it.
+    if (misaligned && !g->retile) make_retile_workspace(g);
+    retile_now = g->retile && (misaligned || row_bytes % 16 != 0);
+  }
+  if (retile_now) {
     TransposeParams t;
     t.batch = g->B;
     // (1-bit rows are moved as 32-bit words)
@@ -428,11 +453,9 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
 }
 
 int ccglib_gemm_destroy(ccglib_gemm_t g) {
-  if (g && (g->workspace || g->aux.stream)) {
+  if (g && g->workspace) {
     DeviceGuard guard(g->device);
-    if (g->aux.stream) (void)hipStreamSynchronize(g->aux.stream);
-    release_aux(&g->aux);
-    if (g->workspace) (void)hipFree(g->workspace);   // waits for the kernels that still use it
+    (void)hipFree(g->workspace);   // waits for the kernels that still use it
   }
   delete g;
   return CCGLIB_OK;
@@ -570,8 +593,8 @@ int ccglib_packing_run(ccglib_packing_t k, const void *d_input, void *d_output) 
   hipError_t e;
   if (k->direction == kForward) {
     e = launch_pack_bits(static_cast<const unsigned char *>(d_input),
-                         static_cast<unsigned *>(d_output), k->N, k->axis == kInterleaved,
-                         k->stream);
+                         static_cast<unsigned *>(d_output), k->N / k->segments,
+                         k->axis == kInterleaved, k->stream, k->segments);
   } else {
     e = launch_unpack_bits(static_cast<const unsigned *>(d_input),
                            static_cast<unsigned char *>(d_output), k->N, k->stream);
@@ -648,6 +671,7 @@ int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
     if (p->d_b_trans) (void)hipFree(p->d_b_trans);
   }
   destroy_host_lanes(p);
+  ccglib_pipeline_destroy(p->unfused);
   ccglib_packing_destroy(p->pack_a);
   ccglib_packing_destroy(p->pack_b);
   ccglib_transpose_destroy(p->trans_a);
@@ -657,11 +681,18 @@ int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
   return CCGLIB_OK;
 }
 
-int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
-                           int device, void *stream, int input_complex_axis_location,
-                           int output_complex_axis_location, int a_mem_order, int b_mem_order,
-                           int c_mem_order, int input_type, int output_type, int variant,
-                           float alpha_re, float alpha_im, float beta_re, float beta_im) {
+}  // extern "C"
+
+namespace {
+
+// allow_fused: the GEMM may read interleaved input in place (false for the
+// pipeline that stands in for it when the caller's buffers are not aligned).
+int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
+                    int device, void *stream, int input_complex_axis_location,
+                    int output_complex_axis_location, int a_mem_order, int b_mem_order,
+                    int c_mem_order, int input_type, int output_type, int variant,
+                    float alpha_re, float alpha_im, float beta_re, float beta_im,
+                    bool allow_fused) {
   if (!pipeline) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null handle pointer");
   *pipeline = nullptr;
   if (!is_enum01(input_complex_axis_location) || !is_enum01(variant)) {
@@ -704,7 +735,7 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   // smaller price while M N / (M + N) stays below about 2800 (16-bit) or 3000
   // (8-bit input), from the measured rates of the kernels involved.
   const double mn_over_sum = (M + N) ? (double)M * (double)N / (double)(M + N) : 0.0;
-  const bool fused = !packing && input_complex_axis_location == kInterleaved && K > 0 &&
+  const bool fused = allow_fused && !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&
                      (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2800.0 : 3000.0));
   // The reference transposes for the opt variant only (:53) and hands interleaved
@@ -714,8 +745,10 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   const bool basic_needs_tiles = !packing && variant == kBasic &&
                                  input_complex_axis_location == kInterleaved && !fused;
   const bool transposing = ((variant == kOpt) && !fused) || basic_needs_tiles;
-  // Packing already moves all real samples in front of all imaginary ones
-  // (over the whole buffer), so what follows it sees planar data.
+  // Packing moves the real samples of every batch in front of its imaginary ones
+  // (below), so what follows it sees planar data. (The reference hands
+  // input_complex_axis_location to its Transpose here too,
+  // src/pipeline/Pipeline.cpp:78-84, which then de-interleaves packed words.)
   const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
   do {
     if (packing && input_complex_axis_location == kPlanar && B && M && N && K % 32 == 0) {
@@ -733,7 +766,7 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
         // GEMM object owns and frees it)
         const size_t bytes = gemm_int1_tiles_bytes(B, M, N, K);
         DeviceGuard guard(device);
-        if (bytes && bytes <= int1_workspace_cap() && guard.status() == hipSuccess &&
+        if (bytes && bytes <= kInt1TilesCap && guard.status() == hipSuccess &&
             hipMalloc(&p->gemm->workspace, bytes) == hipSuccess) {
           p->gemm->workspace_bytes = bytes;
         } else {
@@ -758,6 +791,20 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
       if ((rc = ccglib_packing_create(&p->pack_b, num_b, kForward, device, stream,
                                       input_complex_axis_location)))
         break;
+      if (input_complex_axis_location == kInterleaved && B > 1) {
+        // The reference packs the whole buffer as one (kernels/packing_kernel.cu:15-22:
+        // all real bits of all batches, then all imaginary bits), which is the
+        // planar layout [B][2][rows][K] that the next steps read only for B = 1.
+        // Here every batch is packed on its own; that needs whole words per plane.
+        if ((M * K) % 32 != 0 || (N * K) % 32 != 0) {
+          rc = fail(CCGLIB_ERROR_UNSUPPORTED,
+                    "1-bit interleaved input with several batches needs M*K and N*K to be "
+                    "multiples of 32 (got M=%zu N=%zu K=%zu)", M, N, K);
+          break;
+        }
+        p->pack_a->segments = B;
+        p->pack_b->segments = B;
+      }
       DeviceGuard guard(device);
       hipError_t e = hipMalloc(&p->d_a_packed, ceil_div(num_a, 32) * 4 + 16);
       if (e == hipSuccess) e = hipMalloc(&p->d_b_packed, ceil_div(num_b, 32) * 4 + 16);
@@ -792,6 +839,7 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
                             c_mem_order, a_mem_order, b_mem_order, alpha_re, alpha_im, beta_re,
                             beta_im);  // :102-105
     if (rc == CCGLIB_OK) p->gemm->input_interleaved = fused;
+    p->fused = fused;
   } while (false);
   if (rc != CCGLIB_OK) {
     const std::string keep = g_last_error;
@@ -803,10 +851,37 @@ int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size
   return CCGLIB_OK;
 }
 
+}  // namespace
+
+extern "C" {
+
+int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
+                           int device, void *stream, int input_complex_axis_location,
+                           int output_complex_axis_location, int a_mem_order, int b_mem_order,
+                           int c_mem_order, int input_type, int output_type, int variant,
+                           float alpha_re, float alpha_im, float beta_re, float beta_im) {
+  return pipeline_create(pipeline, B, M, N, K, device, stream, input_complex_axis_location,
+                         output_complex_axis_location, a_mem_order, b_mem_order, c_mem_order,
+                         input_type, output_type, variant, alpha_re, alpha_im, beta_re, beta_im,
+                         true);
+}
+
 int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, void *d_c) {
   if (!p) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null pipeline handle");
   int rc;
   const void *a = d_a, *b = d_b;
+  if (p->fused && d_a && d_b && ((uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0)) {
+    // The GEMM's copies to LDS need 16-byte aligned rows; the transposes take any
+    // element-aligned address. The pipeline that runs them is created here, once
+    // (the one allocation a device Run may make), and kept.
+    if (!p->unfused) {
+      rc = pipeline_create(&p->unfused, p->B, p->M, p->N, p->K, p->device, p->stream, p->in_axis,
+                           p->c_axis, p->a_order, p->b_order, p->c_order, p->type_in, p->type_out,
+                           p->variant, p->alpha_re, p->alpha_im, p->beta_re, p->beta_im, false);
+      if (rc != CCGLIB_OK) return rc;
+    }
+    return ccglib_pipeline_run(p->unfused, d_a, d_b, d_c);
+  }
   if (p->int1_direct) {
     ccglib_gemm *g = p->gemm;
     if (!d_a || !d_b || !d_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
@@ -838,19 +913,15 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
 namespace {
 
 // Batches per chunk of the overlapped host path, or 0 when the problem is run
-// in one piece: a single batch, less than 8 MiB to move, or 1-bit interleaved
-// input (its packing moves the real samples of the *whole* buffer in front,
-// src/pipeline/Pipeline.cpp:111-114 with kernels/packing_kernel.cu:15-22, so a
-// batch is not a contiguous piece of work there). Chunks of about 32 MiB keep
-// copies in both directions in flight at once (sizes from 8 to 64 MiB measured
-// the same, 128 MiB 7 % slower);
-// CCGLIB_AMD_HOST_CHUNK_BYTES overrides that size.
+// in one piece: a single batch or less than 8 MiB to move. Chunks of about
+// 32 MiB keep copies in both directions in flight at once (sizes from 8 to
+// 64 MiB measured the same, 128 MiB 7 % slower);
+// the option CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES overrides that size.
 size_t host_chunk_batches(const ccglib_pipeline *p, size_t bytes_total) {
-  if (p->B < 2 || (p->type_in == kInt1 && p->in_axis == kInterleaved)) return 0;
+  if (p->B < 2) return 0;
   size_t target = (size_t)32 << 20;
-  const char *env = std::getenv("CCGLIB_AMD_HOST_CHUNK_BYTES");
-  if (env && *env) {
-    target = std::max<size_t>(1, std::strtoull(env, nullptr, 10));
+  if (g_options[CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES]) {
+    target = g_options[CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES];
   } else if (bytes_total < ((size_t)8 << 20)) {
     return 0;
   }
@@ -860,7 +931,7 @@ size_t host_chunk_batches(const ccglib_pipeline *p, size_t bytes_total) {
 }
 
 // Creates the lanes of the chunked host path; an object whose chunk size
-// changed (the environment variable) gets new ones.
+// changed (the option) gets new ones.
 int make_host_lanes(ccglib_pipeline *p, size_t chunk, size_t bytes_a, size_t bytes_b,
                     size_t bytes_c) {
   constexpr int kLanes = ccglib_pipeline::kHostLanes;

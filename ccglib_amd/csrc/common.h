@@ -20,9 +20,6 @@ enum ValueType : int {
   kFloat16 = 5,
   kFloat32 = 6
 };
-// Internal operand type of the MFMA path of the 1-bit GEMM: one fp4 (e2m1)
-// value of +1, -1 or 0 per sample. Never crosses the C ABI.
-enum : int { kFp4Sign = 100 };
 enum : int { kPlanar = 0, kInterleaved = 1 };
 enum : int { kForward = 0, kBackward = 1 };
 enum : int { kRowMajor = 0, kColMajor = 1 };
@@ -42,7 +39,6 @@ inline size_t ceil_div(size_t a, size_t b) { return a / b + (a % b != 0); }
 inline int bits_of(int type) {
   switch (type) {
     case kInt1: return 1;
-    case kFp4Sign: return 4;
     case kFloat8e4m3:
     case kFloat8e5m2: return 8;
     case kBfloat16:
@@ -55,15 +51,6 @@ inline int bits_of(int type) {
 
 // K values (samples) held by one 64-byte tile row.
 inline int k_per_tile(int type_in) { return kTileRowBytes * 8 / bits_of(type_in); }
-
-// A second stream with the events to fork from and join into the caller's
-// stream: work queued there may run beside the kernels on the caller's stream.
-struct GemmAux {
-  static constexpr int kMaxJoins = 8;
-  hipStream_t stream = nullptr;
-  hipEvent_t fork = nullptr;
-  hipEvent_t join[kMaxJoins] = {};
-};
 
 // Problem description for one GEMM launch, in kernel terms. The kernel
 // computes D[y][x] = sum_k X[x][k] * Y[y][k] with x the contiguous output
@@ -90,27 +77,22 @@ struct GemmParams {
   int c_interleaved;    // 0 planar, 1 interleaved
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta;
-  // 1-bit GEMM only: device memory for the operands expanded to fp4 (may be null)
+  // 1-bit pipeline only: device memory for both operands in the tiled 1-bit
+  // layout, which the caller's bytes are packed into (may be null)
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
-  // 1-bit GEMM only: where the expansion of later batches may run while earlier
-  // batches are multiplied (may be null: everything on the one stream)
-  const GemmAux *aux = nullptr;
-  // 1-bit GEMM only: the MFMA kernel may take the packed words as they are
-  // (no expanded copy) when their layout allows it
+  // 1-bit GEMM only: the MFMA kernel may multiply the packed words (0: the
+  // vector-ALU kernel runs whatever the layout)
   int int1_direct = 1;
 };
 
-// Bytes of workspace with which the 1-bit GEMM of this size runs in one pass
-// from an fp4 copy of its operands.
-size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k);
 // Bytes of both operands in the tiled 1-bit layout (what the pipeline packs the
 // caller's bytes into when the GEMM multiplies the packed words as they are).
 size_t gemm_int1_tiles_bytes(size_t batch, size_t m, size_t n, size_t k);
 
 // 1-bit GEMM whose operands p.x / p.y are one byte per sample, planar
-// [batch][2][rows][k] (the pipeline's input): expanded straight into the
-// workspace and multiplied on the fp4 MFMA. Only when gemm_int1_can_take_bytes.
+// [batch][2][rows][k] (the pipeline's input): packed straight into 1-bit tiles
+// in the workspace and multiplied on the fp4 MFMA. Only when gemm_int1_can_take_bytes.
 bool gemm_int1_can_take_bytes(const GemmParams &p);
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream);
 
@@ -127,8 +109,11 @@ struct TransposeParams {
 };
 hipError_t launch_transpose(const TransposeParams &p, hipStream_t stream);
 
+// Interleaved input may be `segments` buffers of n samples each, one after the
+// other, each packed on its own into ceil(n / 32) words (real bits, then
+// imaginary bits).
 hipError_t launch_pack_bits(const unsigned char *in, unsigned *out, size_t n,
-                            int interleaved, hipStream_t stream);
+                            int interleaved, hipStream_t stream, size_t segments = 1);
 hipError_t launch_unpack_bits(const unsigned *in, unsigned char *out, size_t n,
                               hipStream_t stream);
 

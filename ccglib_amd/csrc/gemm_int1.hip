@@ -3,11 +3,11 @@
 // Stands in for the reference's int1 wmma_complex_gemm_basic / _opt
 // (kernels/gemm_kernel_int1.cu:64-196, :198-356), which exist for NVIDIA's
 // binary tensor-core op only; gfx950 has no 1-bit matrix instruction. This file
-// holds the launcher, which picks one of three ways to the same integers:
+// holds the launcher, which picks one of two ways to the same integers:
 //  * the fp4 MFMA kernel on the packed words as they are (in the file of the MFMA
-//    kernels; tiled operands and planar rows of whole 16-byte chunks),
-//  * the same MFMA on a copy of the operands expanded to fp4 (expand_* below),
-//  * XOR + population count on the vector ALU (complex_gemm_int1 below),
+//    kernels; tiled operands and planar rows of whole aligned 16-byte chunks),
+//  * XOR + population count on the vector ALU (complex_gemm_int1 below; the
+//    fallback for everything else),
 // and the kernel that packs one byte per sample straight into 1-bit tiles for
 // the pipeline.
 //
@@ -185,163 +185,7 @@ hipError_t launch_loader(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// ---------------------------------------------------------------------------
-// MFMA path. CDNA4 has no 1-bit MFMA, but its fp4 (e2m1) MFMA runs at twice the
-// fp8 rate and +-1 products summed in fp32 are exact integers (up to 2^24), so
-// the packed operands are first expanded - one nibble per sample: 0x2 = +1.0,
-// 0xA = -1.0, 0x0 = 0.0 for the positions past K - into the tiled layout of
-// the MFMA kernel ([batch][rows/128][K/128][2][128 rows][64 bytes]), and the
-// complex GEMM then runs on the matrix cores. With +-1 values the four real
-// products give K - 2 popc(x ^ y) directly, and the zeros make the padding
-// drop out, which is what the reference's K_PADDING correction computes.
-// (Bits past K inside the last word are ignored here; the popcount kernel and
-// the reference count them and so require them to be zero, which Packing
-// guarantees. For such input both paths give the same result.)
-// ---------------------------------------------------------------------------
 typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
-
-// 8 bits -> bit i at position 4 i
-__device__ __forceinline__ unsigned spread8(unsigned x) {
-  x = (x | (x << 12)) & 0x000f000fu;
-  x = (x | (x << 6)) & 0x03030303u;
-  x = (x | (x << 3)) & 0x11111111u;
-  return x;
-}
-
-// 32 samples -> 32 nibbles: 0x2 | bit << 3 where the sample exists, 0 where it
-// does not (bits of `word` outside `valid` are zero). Whole words, which is all
-// of them except at the end of K, skip the second spread: the kernels are close
-// to being bound by this arithmetic rather than by their stores.
-__device__ __forceinline__ uint4_t nibbles_of(unsigned word, unsigned valid) {
-  uint4_t o;
-  if (valid == 0xffffffffu) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) o[q] = (spread8((word >> (8 * q)) & 0xffu) << 3) | 0x22222222u;
-  } else {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      o[q] = (spread8((word >> (8 * q)) & 0xffu) << 3) | (spread8((valid >> (8 * q)) & 0xffu) << 1);
-    }
-  }
-  return o;
-}
-
-// A thread takes word c (of four) of each of the four 128-sample K tiles that a
-// 64-byte row of the 1-bit layout spans: four 4-byte loads in flight per thread
-// (with one, the kernel is bound by the latency of its reads), and every store
-// instruction of a wave writes 16 rows x 64 bytes = 1 KiB contiguous.
-// TILED: the source is the 1-bit tiled layout (tiles of 512 samples); otherwise
-// planar rows of k_words words.
-template <bool TILED>
-__global__ __launch_bounds__(256) void expand_int1_to_fp4(const char *__restrict__ src,
-                                                          char *__restrict__ dst, unsigned rows, unsigned row_tiles,
-                                                          unsigned k, unsigned k1_tiles,
-                                                          unsigned k4_tiles, unsigned k_words) {
-  // blockIdx.x: (batch, row tile, source K tile of 512 samples); blockIdx.y: (plane, half of the 128 rows)
-  const unsigned c = threadIdx.x & 3, row = (blockIdx.y & 1) * 64 + (threadIdx.x >> 2);
-  const unsigned plane = blockIdx.y >> 1;
-  const unsigned kt1 = blockIdx.x % k1_tiles;
-  const unsigned rest = blockIdx.x / k1_tiles;
-  const unsigned rt = rest % row_tiles;
-  const size_t b = rest / row_tiles;
-  unsigned w[4] = {0, 0, 0, 0};
-  if constexpr (TILED) {
-    const unsigned *p = reinterpret_cast<const unsigned *>(
-                            src + ((b * row_tiles + rt) * k1_tiles + kt1) * kTileBytes +
-                            plane * kTilePlaneBytes + row * kTileRowBytes) + c;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) w[s] = p[4 * s];
-  } else {
-    const unsigned r = rt * kTileRows + row;
-    if (r < rows) {
-      const unsigned *p = reinterpret_cast<const unsigned *>(src) +
-                          ((b * 2 + plane) * rows + r) * (size_t)k_words + 16 * kt1 + c;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        if (16 * kt1 + 4 * s + c < k_words) w[s] = p[4 * s];
-      }
-    }
-  }
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const unsigned k4 = 4 * kt1 + s;          // K tile of the expanded layout (128 samples)
-    if (k4 >= k4_tiles) break;
-    // samples of this word that exist: the others become 0.0
-    const unsigned first = k4 * 128 + 32 * c;
-    const unsigned n = first >= k ? 0u : (k - first >= 32 ? 32u : k - first);
-    const unsigned valid = n == 32 ? 0xffffffffu : ((1u << n) - 1u);
-    const unsigned ws = w[s] & valid;
-    const uint4_t o = nibbles_of(ws, valid);
-    __builtin_nontemporal_store(
-        o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
-                                       plane * kTilePlaneBytes + row * kTileRowBytes + 16 * c));
-  }
-}
-
-// The same expansion straight from one byte per sample (the pipeline's input:
-// any non-zero byte is a 1, kernels/packing_kernel.cu:14-22), which saves the
-// packed and the transposed intermediate of the pack -> transpose -> expand
-// sequence. Planar input [batch][2][rows][k]; a thread takes 32 samples of each
-// of four K tiles (eight 16-byte loads in flight) and writes four 16-byte pieces;
-// every store instruction of a wave writes 1 KiB contiguous.
-__device__ __forceinline__ unsigned nonzero_bits_of4(unsigned x) {   // 4 bytes -> 4 bits
-  const unsigned nz = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
-  return (((nz >> 7) * 0x00204081u) >> 21) & 0xfu;
-}
-__device__ __forceinline__ unsigned nonzero_bits_of16(uint4_t v) {
-  return nonzero_bits_of4(v[0]) | (nonzero_bits_of4(v[1]) << 4) | (nonzero_bits_of4(v[2]) << 8) |
-         (nonzero_bits_of4(v[3]) << 12);
-}
-
-template <bool VEC>
-__global__ __launch_bounds__(256) void expand_bytes_to_fp4(const unsigned char *__restrict__ src,
-                                                           char *__restrict__ dst, unsigned rows,
-                                                           unsigned row_tiles, unsigned k,
-                                                           unsigned k4_tiles) {
-  // blockIdx: x = group of four K tiles of 128 samples (512 bytes of a row), y = block of 64
-  // rows, z = (batch, plane). A wave takes 16 rows, four at a time: lane = (row of the four,
-  // 32-sample piece of the 512), so that a load instruction reads four runs of 512
-  // contiguous bytes; a thread has eight 16-byte loads in flight (four rows, two each) and
-  // writes four 16-byte pieces (a store instruction writes 256 contiguous bytes in each of
-  // four K tiles).
-  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const unsigned piece = lane & 15, s = piece >> 2, c = piece & 3;
-  const unsigned rt = blockIdx.y >> 1;
-  const size_t b = blockIdx.z >> 1;
-  const unsigned plane = blockIdx.z & 1;
-  const unsigned k4 = 4 * blockIdx.x + s;
-  const unsigned k0 = k4 * 128 + c * 32;
-  unsigned row_in_tile[4], n[4];
-  const unsigned char *row_ptr[4];
-  uint4_t v[4][2];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    row_in_tile[q] = (blockIdx.y & 1) * 64 + wave * 16 + q * 4 + (lane >> 4);
-    const unsigned r = rt * kTileRows + row_in_tile[q];
-    row_ptr[q] = src + ((b * 2 + plane) * rows + (r < rows ? r : 0)) * (size_t)k;
-    n[q] = (r < rows && k0 < k) ? (k - k0 < 32 ? k - k0 : 32) : 0;
-    if (VEC && n[q] == 32) {
-      v[q][0] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0));
-      v[q][1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(row_ptr[q] + k0) + 1);
-    }
-  }
-  if (k4 >= k4_tiles) return;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    unsigned bits;
-    if (VEC && n[q] == 32) {
-      bits = nonzero_bits_of16(v[q][0]) | (nonzero_bits_of16(v[q][1]) << 16);
-    } else {
-      bits = 0;
-      for (unsigned i = 0; i < n[q]; ++i) bits |= (row_ptr[q][k0 + i] != 0 ? 1u : 0u) << i;
-    }
-    const unsigned valid = n[q] == 32 ? 0xffffffffu : ((1u << n[q]) - 1u);
-    const uint4_t o = nibbles_of(bits, valid);
-    __builtin_nontemporal_store(
-        o, reinterpret_cast<uint4_t *>(dst + ((b * row_tiles + rt) * k4_tiles + k4) * kTileBytes +
-                                       plane * kTilePlaneBytes + row_in_tile[q] * kTileRowBytes + 16 * c));
-  }
-}
 
 // One byte per sample straight into the tiled 1-bit layout that the opt variant
 // reads ([batch][rows/128][K/512][2][128 rows][64 bytes]; rows and samples past
@@ -432,64 +276,6 @@ __global__ __launch_bounds__(256) void pack_bytes_to_tiles(const unsigned char *
 // Largest K for which every partial sum (at most 2 K in magnitude) is exact in fp32.
 constexpr unsigned kMaxMfmaK = 1u << 22;
 
-// Batches per group when the expansion of one group of batches is to overlap
-// the multiplication of the previous one (the expansion is bound by memory
-// bandwidth, the multiplication by the matrix cores): the fewest batches that
-// give every compute unit a C tile, at most GemmAux::kMaxJoins groups; the
-// whole batch when that leaves fewer than two groups or there is no second
-// stream.
-size_t overlap_group(const GemmParams &p) {
-  if (!p.aux || !p.aux->stream) return p.batch;
-  const size_t tiles_per_batch = ceil_div(p.nx, 256) * ceil_div(p.ny, 128);
-  size_t group = ceil_div(256, tiles_per_batch);
-  group = std::max(group, ceil_div(p.batch, GemmAux::kMaxJoins));
-  return 2 * group <= p.batch ? group : p.batch;
-}
-
-// Expands (expand(b0, nb, ws_x, ws_y, stream)) and multiplies the batches in
-// groups of `group`; the workspace holds the groups one after the other when
-// `ws_advances`, else every group uses its start. With a second stream (only
-// when the workspace advances, so that no group overwrites what another still
-// needs) all expansions are queued there and each multiplication waits for its
-// own group's.
-template <typename Expand>
-hipError_t run_groups(const GemmParams &p, hipStream_t stream, size_t group, bool ws_advances,
-                      unsigned k4_tiles, Expand &&expand) {
-  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
-  const size_t y_bytes = (size_t)p.y_tiles * k4_tiles * kTileBytes;
-  const bool overlap = ws_advances && p.aux && p.aux->stream && group < p.batch &&
-                       ceil_div(p.batch, group) <= (size_t)GemmAux::kMaxJoins;
-  hipStream_t expand_stream = overlap ? p.aux->stream : stream;
-  if (overlap) {
-    // the operands may still be being written on the caller's stream
-    if (hipError_t e = hipEventRecord(p.aux->fork, stream)) return e;
-    if (hipError_t e = hipStreamWaitEvent(p.aux->stream, p.aux->fork, 0)) return e;
-  }
-  char *ws = static_cast<char *>(p.workspace);
-  int gi = 0;
-  for (size_t b0 = 0; b0 < p.batch; b0 += group, ++gi) {
-    const size_t nb = (p.batch - b0 < group) ? p.batch - b0 : group;
-    char *ws_x = ws, *ws_y = ws + nb * x_bytes;
-    if (ws_advances) ws += nb * (x_bytes + y_bytes);
-    if (hipError_t e = expand(b0, nb, ws_x, ws_y, expand_stream)) return e;
-    if (overlap) {
-      if (hipError_t e = hipEventRecord(p.aux->join[gi], p.aux->stream)) return e;
-      if (hipError_t e = hipStreamWaitEvent(stream, p.aux->join[gi], 0)) return e;
-    }
-    GemmParams q = p;
-    q.x = ws_x;
-    q.y = ws_y;
-    q.c = static_cast<char *>(p.c) + b0 * 2 * (size_t)p.nx * p.ny * 4;
-    q.batch = (unsigned)nb;
-    q.k_tiles = k4_tiles;
-    q.type_in = kFp4Sign;
-    q.variant = kOpt;
-    q.input_interleaved = 0;
-    if (hipError_t e = launch_gemm_mfma(q, stream)) return e;
-  }
-  return hipGetLastError();
-}
-
 // The packed words as they are: tiled operands always (16-byte aligned, which
 // the caller has checked), planar rows when they are whole aligned 16-byte
 // chunks (K a multiple of 128).
@@ -528,108 +314,43 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
     }
     return hipSuccess;
   }
-  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return hipSuccess;
-  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
-  const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
-  const unsigned k_words = (unsigned)ceil_div(p.k, 32);
-  const size_t x_bytes = (size_t)p.x_tiles * k4_tiles * kTileBytes;   // per batch, expanded
-  const size_t y_bytes = (size_t)p.y_tiles * k4_tiles * kTileBytes;
-  const size_t fits = p.workspace_bytes / (x_bytes + y_bytes);
-  if (fits == 0) return hipSuccess;
-  const bool tiled = (p.variant == kOpt);
-  if (((uintptr_t)p.x | (uintptr_t)p.y) % 4 != 0) return hipSuccess;
-  const size_t x_src = tiled ? (size_t)p.x_tiles * k1_tiles * kTileBytes : (size_t)2 * p.nx * k_words * 4;
-  const size_t y_src = tiled ? (size_t)p.y_tiles * k1_tiles * kTileBytes : (size_t)2 * p.ny * k_words * 4;
-  auto expand = [&](size_t b0, size_t nb, char *ws_x, char *ws_y, hipStream_t s) -> hipError_t {
-    for (int which = 0; which < 2; ++which) {
-      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
-      const char *src = static_cast<const char *>(which ? p.y : p.x) + b0 * (which ? y_src : x_src);
-      char *dst = which ? ws_y : ws_x;
-      const size_t blocks = nb * row_tiles * k1_tiles;
-      if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-      const dim3 grid((unsigned)blocks, 4);
-      if (tiled) {
-        hipLaunchKernelGGL(expand_int1_to_fp4<true>, grid, dim3(256), 0, s, src, dst, rows,
-                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
-      } else {
-        hipLaunchKernelGGL(expand_int1_to_fp4<false>, grid, dim3(256), 0, s, src, dst, rows,
-                           row_tiles, p.k, k1_tiles, k4_tiles, k_words);
-      }
-    }
-    return hipSuccess;
-  };
-  // the whole problem in the workspace: groups chosen for overlap, laid out one
-  // after the other; a smaller workspace: as many batches at a time as fit
-  const bool whole = fits >= p.batch;
-  const size_t group = whole ? overlap_group(p) : fits;
-  if (hipError_t e = run_groups(p, stream, group, whole, k4_tiles, expand)) return e;
-  *done = true;
-  return hipSuccess;
+  return hipSuccess;   // not done: the caller runs the vector-ALU kernel
 }
 
 }  // namespace
 
 bool gemm_int1_can_take_bytes(const GemmParams &p) {
-  if (!p.workspace || p.k == 0 || p.k > kMaxMfmaK) return false;
-  const size_t need = p.int1_direct ? gemm_int1_tiles_bytes(p.batch, p.nx, p.ny, p.k)
-                                    : gemm_int1_workspace_bytes(p.batch, p.nx, p.ny, p.k);
-  if (p.workspace_bytes < need) return false;
+  if (!p.int1_direct || !p.workspace || p.k == 0 || p.k > kMaxMfmaK) return false;
+  if (p.workspace_bytes < gemm_int1_tiles_bytes(p.batch, p.nx, p.ny, p.k)) return false;
   return p.batch <= 32767 && 16 * (size_t)p.x_tiles <= 65535 && 16 * (size_t)p.y_tiles <= 65535;
 }
 
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) {
   if (!gemm_int1_can_take_bytes(p)) return hipErrorInvalidValue;
-  if (p.int1_direct) {
-    // pack into the tiled 1-bit layout and multiply the packed words as they are
-    const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
-    const size_t x_bytes = (size_t)p.batch * p.x_tiles * k1_tiles * kTileBytes;
-    char *ws_x = static_cast<char *>(p.workspace), *ws_y = ws_x + x_bytes;
-    for (int which = 0; which < 2; ++which) {
-      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
-      const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
-      const dim3 grid((unsigned)ceil_div(k1_tiles, 4), (kTileRows / (2 * kPackLoads)) * row_tiles, 2 * p.batch);
-      const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
-      if (vec) {
-        hipLaunchKernelGGL(pack_bytes_to_tiles<true>, grid, dim3(256), 0, stream, src,
-                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
-      } else {
-        hipLaunchKernelGGL(pack_bytes_to_tiles<false>, grid, dim3(256), 0, stream, src,
-                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
-      }
+  // pack into the tiled 1-bit layout and multiply the packed words as they are
+  const unsigned k1_tiles = (unsigned)ceil_div(p.k, 512);
+  const size_t x_bytes = (size_t)p.batch * p.x_tiles * k1_tiles * kTileBytes;
+  char *ws_x = static_cast<char *>(p.workspace), *ws_y = ws_x + x_bytes;
+  for (int which = 0; which < 2; ++which) {
+    const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
+    const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
+    const dim3 grid((unsigned)ceil_div(k1_tiles, 4), (kTileRows / (2 * kPackLoads)) * row_tiles, 2 * p.batch);
+    const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
+    if (vec) {
+      hipLaunchKernelGGL(pack_bytes_to_tiles<true>, grid, dim3(256), 0, stream, src,
+                         which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
+    } else {
+      hipLaunchKernelGGL(pack_bytes_to_tiles<false>, grid, dim3(256), 0, stream, src,
+                         which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
     }
-    if (hipError_t e = hipGetLastError()) return e;
-    GemmParams q = p;
-    q.x = ws_x;
-    q.y = ws_y;
-    q.variant = kOpt;
-    q.k_tiles = k1_tiles;
-    return launch_gemm_mfma(q, stream);
   }
-  const unsigned k4_tiles = (unsigned)ceil_div(p.k, 128);
-  auto expand = [&](size_t b0, size_t nb, char *ws_x, char *ws_y, hipStream_t s) -> hipError_t {
-    for (int which = 0; which < 2; ++which) {
-      const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
-      const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x) +
-                                 b0 * 2 * (size_t)rows * p.k;
-      char *dst = which ? ws_y : ws_x;
-      const dim3 grid((unsigned)ceil_div(k4_tiles, 4), 2 * row_tiles, 2 * (unsigned)nb);
-      const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
-      if (vec) {
-        hipLaunchKernelGGL(expand_bytes_to_fp4<true>, grid, dim3(256), 0, s, src, dst, rows,
-                           row_tiles, p.k, k4_tiles);
-      } else {
-        hipLaunchKernelGGL(expand_bytes_to_fp4<false>, grid, dim3(256), 0, s, src, dst, rows,
-                           row_tiles, p.k, k4_tiles);
-      }
-    }
-    return hipSuccess;
-  };
-  return run_groups(p, stream, overlap_group(p), true, k4_tiles, expand);
-}
-
-size_t gemm_int1_workspace_bytes(size_t batch, size_t m, size_t n, size_t k) {
-  if (k == 0 || k > kMaxMfmaK) return 0;
-  return batch * (ceil_div(m, kTileRows) + ceil_div(n, kTileRows)) * ceil_div(k, 128) * kTileBytes;
+  if (hipError_t e = hipGetLastError()) return e;
+  GemmParams q = p;
+  q.x = ws_x;
+  q.y = ws_y;
+  q.variant = kOpt;
+  q.k_tiles = k1_tiles;
+  return launch_gemm_mfma(q, stream);
 }
 
 size_t gemm_int1_tiles_bytes(size_t batch, size_t m, size_t n, size_t k) {

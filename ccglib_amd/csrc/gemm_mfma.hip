@@ -8,17 +8,21 @@
 // products per complex product (gemm_kernel_float.cu:293-303); everything
 // else is laid out for 64-wide wavefronts:
 //
-//  * One block owns a BX x BY patch of C and walks K in tiles of 64 bytes.
-//    For the tiled (opt) layout the tiles go global -> LDS directly
-//    (global_load_lds_dwordx4) through a ring of LDS slots, two iterations
-//    ahead of the math; the planar (basic) layouts are staged through
-//    registers, which is where their bounds checks and zero fill happen.
-//  * LDS rows are 64 bytes; the 16-byte chunk index is XORed with
-//    (row >> 1) & 3, which makes both the linear 16-byte writes and the
-//    16-row fragment reads free of bank conflicts on this LDS.
-//  * 16x16x32 MFMA (16x16x128 for fp8). The operand whose rows run along the
-//    contiguous axis of C is the MFMA "A" operand, so each lane ends up with
-//    four consecutive C elements and stores them with one 16-byte write.
+//  * One persistent block owns a sequence of BX x BY patches of C and walks K in
+//    tiles of 64 bytes per row. Tiles go global -> LDS directly
+//    (global_load_lds_dwordx4) through a ring of LDS slots, two iterations ahead
+//    of the math: for the tiled (opt) layout, for planar (basic) rows that are
+//    whole aligned 16-byte chunks, and for the pipeline's interleaved rows. Only
+//    planar rows that are neither (and have no tiled copy) are staged through
+//    registers by a second kernel, whose element-wise loads do their bounds
+//    checks and zero fill.
+//  * LDS rows are 64 bytes with the 16-byte chunk index XORed by a function of
+//    the row that suits the fragment shape of the MFMA in use (measured free of
+//    bank conflicts; see complex_gemm_mfma_dtl).
+//  * 16-bit and 32-bit input: 16x16x32 (16x16x4 for fp32) MFMA; fp8: the
+//    32x32x64 f8f6f4 MFMA, which runs at twice the rate of the legacy fp8
+//    instruction; 1-bit input: the same instruction on fp4 +-1 values expanded
+//    from the packed words in registers.
 //  * The four products of a complex MAC reuse the same fragments; the minus
 //    sign of Re -= Xi*Yi is a sign-bit flip of the Yi fragment registers.
 //  * Workgroup ids are remapped so that consecutive tiles land on the same
@@ -44,8 +48,7 @@ template <int DT> struct DtypeTraits {
   static constexpr int kElemBytes = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 1
                                     : (DT == kFloat32)                       ? 4
                                                                              : 2;
-  static constexpr unsigned kSignMask = (DT == kFp4Sign)                            ? 0x88888888u
-                                        : (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u
+  static constexpr unsigned kSignMask = (DT == kFloat8e4m3 || DT == kFloat8e5m2) ? 0x80808080u
                                         : (DT == kFloat32)                         ? 0x80000000u
                                                                                    : 0x80008000u;
 };
@@ -133,16 +136,6 @@ __device__ __forceinline__ float16_t_ mfma32(const Fragment32 &a, const Fragment
                                                     __builtin_bit_cast(bf16x8_t, b.v[u]), acc, 0, 0, 0);
     }
     return acc;
-  } else if constexpr (DT == kFp4Sign) {
-    // fp4: 64 values of K are 16 bytes per lane, so the 64-byte row is two
-    // instructions (format code 4; only the low four registers are read)
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int8_t_ av = {a.v[u][0], a.v[u][1], a.v[u][2], a.v[u][3], 0, 0, 0, 0};
-      const int8_t_ bv = {b.v[u][0], b.v[u][1], b.v[u][2], b.v[u][3], 0, 0, 0, 0};
-      acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 0, 0x7f, 0, 0x7f);
-    }
-    return acc;
   } else {
     int8_t_ av, bv;
 #pragma unroll
@@ -159,22 +152,31 @@ __device__ __forceinline__ float16_t_ mfma32(const Fragment32 &a, const Fragment
 }
 
 // Accumulator of one MFMA tile and how the output is spread over a wave, for
-// both MFMA shapes (MS = 16 or 32 rows). A lane holds "pieces" of four
-// consecutive x (the contiguous C axis) at one y:
-//   MS 16: piece (jj, ii) at x = 16 ii + 4 (lane / 16), y = 16 jj + lane % 16
-//   MS 32: piece (jj, ii) at x = 32 (ii / 4) + 8 (ii % 4) + 4 (lane / 32), y = 32 jj + lane % 32
+// both MFMA shapes (MS = 16 or 32 rows) and for the 16-row shape with the
+// operand roles exchanged (kAcc16T: X is the MFMA "B" operand and tile i of a
+// wave holds the columns x = 4 (lane % 16) + i, see complex_gemm_mfma_dtl).
+// A lane holds "pieces" of four consecutive x (the contiguous C axis) at one y:
+//   MS 16:   piece (jj, ii) at x = 16 ii + 4 (lane / 16), y = 16 jj + lane % 16
+//   MS 32:   piece (jj, ii) at x = 32 (ii / 4) + 8 (ii % 4) + 4 (lane / 32), y = 32 jj + lane % 32
+//   kAcc16T: piece (jj, ii) at x = 4 (lane % 16), y = 16 jj + 4 (lane / 16) + ii; its four
+//            elements are register ii of the four tiles of tile row jj
+constexpr int kAcc16T = 116;
 template <int MS> struct AccType { using type = float4_t; };
 template <> struct AccType<32> { using type = float16_t_; };
 
 template <int MS> __device__ __forceinline__ unsigned piece_x(int ii, int lane) {
+  if constexpr (MS == kAcc16T) return (lane & 15) * 4;
   return MS == 16 ? ii * 16 + (lane >> 4) * 4 : (ii >> 2) * 32 + (ii & 3) * 8 + (lane >> 5) * 4;
 }
-template <int MS> __device__ __forceinline__ unsigned piece_y(int jj, int lane) {
+template <int MS> __device__ __forceinline__ unsigned piece_y(int jj, int ii, int lane) {
+  if constexpr (MS == kAcc16T) return jj * 16 + (lane >> 4) * 4 + ii;
   return MS == 16 ? jj * 16 + (lane & 15) : jj * 32 + (lane & 31);
 }
 template <int MS, typename Acc>
 __device__ __forceinline__ float piece_elem(const Acc &acc, int jj, int ii, int e) {
-  if constexpr (MS == 16) {
+  if constexpr (MS == kAcc16T) {
+    return acc[jj][e][ii];
+  } else if constexpr (MS == 16) {
     return acc[jj][ii][e];
   } else {
     return acc[jj][ii >> 2][(ii & 3) * 4 + e];
@@ -235,8 +237,11 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
 // cores wait for the whole queue. Here a wave reads what its first MFMA needs,
 // keeps about three reads in flight ahead of their use, and fetches the Y
 // fragments of the next tile row during the current one.
-template <int DT, int BX, int BY, typename Mid>
-__device__ __forceinline__ void mma_step_ordered(const char *slot, int x_frag_off, int y_frag_off,
+// xo[i] is the lane's offset of the X fragment of tile i. XT: the operand roles
+// of the MFMA are exchanged (Y supplies the instruction's "A" rows, X its "B"
+// columns), which transposes what a lane holds of every 16 x 16 tile.
+template <int DT, int BX, int BY, bool XT, typename Mid>
+__device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&xo)[4], int y_frag_off,
                                                  float4_t (&acc_re)[4][4], float4_t (&acc_im)[4][4],
                                                  Mid &&mid) {
   static_assert(DtypeTraits<DT>::kTilesPerMfma == 1, "one K tile per MFMA");
@@ -245,46 +250,49 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, int x_frag_of
     f.v[0] = *reinterpret_cast<const int4_t *>(slot + off);
     return f;
   };
+  auto mm = [](const Fragment<DT> &x, const Fragment<DT> &y, float4_t acc) {
+    return XT ? mfma<DT>(y, x, acc) : mfma<DT>(x, y, acc);
+  };
   constexpr int ROW16 = 16 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
 #define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
   Fragment<DT> xr[4], xi[4], yr, yi, yin, yr_next, yi_next;
   yr = rd(y_frag_off);
-  xr[0] = rd(x_frag_off);
-  xr[1] = rd(x_frag_off + ROW16);
-  xr[2] = rd(x_frag_off + 2 * ROW16);
+  xr[0] = rd(xo[0]);
+  xr[1] = rd(xo[1]);
+  xr[2] = rd(xo[2]);
   CCGLIB_PIN;
-  acc_re[0][0] = mfma<DT>(xr[0], yr, acc_re[0][0]);
-  xr[3] = rd(x_frag_off + 3 * ROW16);
+  acc_re[0][0] = mm(xr[0], yr, acc_re[0][0]);
+  xr[3] = rd(xo[3]);
   CCGLIB_PIN;
-  acc_re[0][1] = mfma<DT>(xr[1], yr, acc_re[0][1]);
+  acc_re[0][1] = mm(xr[1], yr, acc_re[0][1]);
   yi = rd(y_frag_off + YP);
   CCGLIB_PIN;
-  acc_re[0][2] = mfma<DT>(xr[2], yr, acc_re[0][2]);
-  xi[0] = rd(x_frag_off + XP);
+  acc_re[0][2] = mm(xr[2], yr, acc_re[0][2]);
+  xi[0] = rd(xo[0] + XP);
   CCGLIB_PIN;
-  acc_re[0][3] = mfma<DT>(xr[3], yr, acc_re[0][3]);
-  xi[1] = rd(x_frag_off + XP + ROW16);
+  acc_re[0][3] = mm(xr[3], yr, acc_re[0][3]);
+  xi[1] = rd(xo[1] + XP);
   CCGLIB_PIN;
-  acc_im[0][0] = mfma<DT>(xr[0], yi, acc_im[0][0]);
-  xi[2] = rd(x_frag_off + XP + 2 * ROW16);
+  acc_im[0][0] = mm(xr[0], yi, acc_im[0][0]);
+  xi[2] = rd(xo[2] + XP);
   CCGLIB_PIN;
-  acc_im[0][1] = mfma<DT>(xr[1], yi, acc_im[0][1]);
-  xi[3] = rd(x_frag_off + XP + 3 * ROW16);
+  acc_im[0][1] = mm(xr[1], yi, acc_im[0][1]);
+  xi[3] = rd(xo[3] + XP);
   CCGLIB_PIN;
-  acc_im[0][2] = mfma<DT>(xr[2], yi, acc_im[0][2]);
+  acc_im[0][2] = mm(xr[2], yi, acc_im[0][2]);
   yin = negate<DT>(yi);
   CCGLIB_PIN;
-  acc_im[0][3] = mfma<DT>(xr[3], yi, acc_im[0][3]);
+  acc_im[0][3] = mm(xr[3], yi, acc_im[0][3]);
   yr_next = rd(y_frag_off + ROW16);
   CCGLIB_PIN;
-  acc_re[0][0] = mfma<DT>(xi[0], yin, acc_re[0][0]);
+  acc_re[0][0] = mm(xi[0], yin, acc_re[0][0]);
   yi_next = rd(y_frag_off + YP + ROW16);
   CCGLIB_PIN;
-  acc_im[0][0] = mfma<DT>(xi[0], yr, acc_im[0][0]);
+  acc_im[0][0] = mm(xi[0], yr, acc_im[0][0]);
 #pragma unroll
   for (int i = 1; i < 4; ++i) {
-    acc_re[0][i] = mfma<DT>(xi[i], yin, acc_re[0][i]);
-    acc_im[0][i] = mfma<DT>(xi[i], yr, acc_im[0][i]);
+    acc_re[0][i] = mm(xi[i], yin, acc_re[0][i]);
+    acc_im[0][i] = mm(xi[i], yr, acc_im[0][i]);
   }
   CCGLIB_PIN;
   mid();
@@ -298,26 +306,26 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, int x_frag_of
     // from one MFMA to the next only one of the two operands changes (measured 1-2 %
     // faster on random data than four MFMAs per Y fragment in a row: the part is
     // power limited, and this order toggles fewer operand bits)
-    acc_re[j][0] = mfma<DT>(xr[0], yr, acc_re[j][0]);
-    acc_im[j][0] = mfma<DT>(xr[0], yi, acc_im[j][0]);
-    acc_im[j][1] = mfma<DT>(xr[1], yi, acc_im[j][1]);
-    acc_re[j][1] = mfma<DT>(xr[1], yr, acc_re[j][1]);
+    acc_re[j][0] = mm(xr[0], yr, acc_re[j][0]);
+    acc_im[j][0] = mm(xr[0], yi, acc_im[j][0]);
+    acc_im[j][1] = mm(xr[1], yi, acc_im[j][1]);
+    acc_re[j][1] = mm(xr[1], yr, acc_re[j][1]);
     if (j < 3) yr_next = rd(y_frag_off + (j + 1) * ROW16);
     CCGLIB_PIN;
-    acc_re[j][2] = mfma<DT>(xr[2], yr, acc_re[j][2]);
-    acc_im[j][2] = mfma<DT>(xr[2], yi, acc_im[j][2]);
-    acc_im[j][3] = mfma<DT>(xr[3], yi, acc_im[j][3]);
-    acc_re[j][3] = mfma<DT>(xr[3], yr, acc_re[j][3]);
+    acc_re[j][2] = mm(xr[2], yr, acc_re[j][2]);
+    acc_im[j][2] = mm(xr[2], yi, acc_im[j][2]);
+    acc_im[j][3] = mm(xr[3], yi, acc_im[j][3]);
+    acc_re[j][3] = mm(xr[3], yr, acc_re[j][3]);
     if (j < 3) yi_next = rd(y_frag_off + YP + (j + 1) * ROW16);
     CCGLIB_PIN;
-    acc_im[j][0] = mfma<DT>(xi[0], yr, acc_im[j][0]);
-    acc_re[j][0] = mfma<DT>(xi[0], yin, acc_re[j][0]);
-    acc_re[j][1] = mfma<DT>(xi[1], yin, acc_re[j][1]);
-    acc_im[j][1] = mfma<DT>(xi[1], yr, acc_im[j][1]);
-    acc_im[j][2] = mfma<DT>(xi[2], yr, acc_im[j][2]);
-    acc_re[j][2] = mfma<DT>(xi[2], yin, acc_re[j][2]);
-    acc_re[j][3] = mfma<DT>(xi[3], yin, acc_re[j][3]);
-    acc_im[j][3] = mfma<DT>(xi[3], yr, acc_im[j][3]);
+    acc_im[j][0] = mm(xi[0], yr, acc_im[j][0]);
+    acc_re[j][0] = mm(xi[0], yin, acc_re[j][0]);
+    acc_re[j][1] = mm(xi[1], yin, acc_re[j][1]);
+    acc_im[j][1] = mm(xi[1], yr, acc_im[j][1]);
+    acc_im[j][2] = mm(xi[2], yr, acc_im[j][2]);
+    acc_re[j][2] = mm(xi[2], yin, acc_re[j][2]);
+    acc_re[j][3] = mm(xi[3], yin, acc_re[j][3]);
+    acc_im[j][3] = mm(xi[3], yr, acc_im[j][3]);
     CCGLIB_PIN;
   }
 #undef CCGLIB_PIN
@@ -826,7 +834,7 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
                                                 unsigned y_wave, int lane, const Acc &acc_re,
                                                 const Acc &acc_im) {
   // TX, TY count MFMA tiles; pieces per tile row: 1 (MS 16) or 4 (MS 32)
-  constexpr int NPX = MS == 16 ? TX : TX * 4;
+  constexpr int NPX = MS == 32 ? TX * 4 : TX;
   using Tout = typename OutType<TOUT>::type;
   const unsigned nx = args.nx, ny = args.ny;
   const bool have_alpha = args.have_alpha, have_beta = args.have_beta;
@@ -835,9 +843,9 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
   const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
-    const unsigned y = y_wave + piece_y<MS>(j, lane);
 #pragma unroll
     for (int i = 0; i < NPX; ++i) {
+      const unsigned y = y_wave + piece_y<MS>(j, i, lane);
       const unsigned x = x_wave + piece_x<MS>(i, lane);
       if (y >= ny || x >= nx) continue;
       float re[4], im[4];
@@ -926,7 +934,7 @@ template <int TX, int TY, int MS, typename Acc>
 __device__ __forceinline__ void store_wave_tile_int32(const KernelArgs &args, unsigned b,
                                                       unsigned x_wave, unsigned y_wave, int lane,
                                                       const Acc &acc_re, const Acc &acc_im) {
-  constexpr int NPX = MS == 16 ? TX : TX * 4;
+  constexpr int NPX = MS == 32 ? TX * 4 : TX;
   const unsigned nx = args.nx, ny = args.ny;
   const unsigned ar = (unsigned)(int)args.alpha_re, ai = (unsigned)(int)args.alpha_im;
   const unsigned br = (unsigned)(int)args.beta_re, bi = (unsigned)(int)args.beta_im;
@@ -935,9 +943,9 @@ __device__ __forceinline__ void store_wave_tile_int32(const KernelArgs &args, un
   const bool vec_ok = (nx % 4 == 0) && args.c_vector_ok;
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
-    const unsigned y = y_wave + piece_y<MS>(j, lane);
 #pragma unroll
     for (int i = 0; i < NPX; ++i) {
+      const unsigned y = y_wave + piece_y<MS>(j, i, lane);
       const unsigned x = x_wave + piece_x<MS>(i, lane);
       if (y >= ny || x >= nx) continue;
       unsigned re[4], im[4];
@@ -992,6 +1000,47 @@ __device__ __forceinline__ void store_wave_tile_int32(const KernelArgs &args, un
               p[2 * e + 1] = im[e];
             }
           }
+        }
+      }
+    }
+  }
+}
+
+// Epilogue of the exchanged-roles layout (kAcc16T) for the common case (planar
+// C, beta = 0, wave tile entirely inside C, vector-aligned rows): register e of
+// the four tiles of a tile row are four consecutive x, so a lane writes 16 bytes
+// (8 for fp16 / bf16 C) and a store instruction four whole 256-byte row segments,
+// straight from the accumulators.
+template <int TOUT, int TY>
+__device__ __forceinline__ void store_wave_tile_rows(const KernelArgs &args, unsigned b,
+                                                     unsigned x_wave, unsigned y_wave, int lane,
+                                                     float4_t (&acc_re)[TY][4],
+                                                     float4_t (&acc_im)[TY][4]) {
+  using Tout = typename OutType<TOUT>::type;
+  const unsigned nx = args.nx, ny = args.ny;
+  const bool have_alpha = args.have_alpha;
+  const float ar = args.alpha_re, ai = args.alpha_im;
+  Tout *out = reinterpret_cast<Tout *>(args.c) + (size_t)b * 2 * nx * ny +
+              (size_t)(y_wave + (lane >> 4) * 4) * nx + x_wave + (lane & 15) * 4;
+#pragma unroll
+  for (int plane = 0; plane < 2; ++plane) {
+#pragma unroll
+    for (int j = 0; j < TY; ++j) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float re = acc_re[j][i][e], im = acc_im[j][i][e];
+          v[i] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
+                            : (have_alpha ? ai * re + ar * im : im);
+        }
+        Tout *p = out + (size_t)plane * nx * ny + (size_t)(j * 16 + e) * nx;
+        if constexpr (TOUT == kFloat32) {
+          *reinterpret_cast<float4_t *>(p) = float4_t{v[0], v[1], v[2], v[3]};
+        } else {
+          Tout t[4] = {(Tout)v[0], (Tout)v[1], (Tout)v[2], (Tout)v[3]};
+          *reinterpret_cast<ushort4_t *>(p) = __builtin_bit_cast(ushort4_t, t);
         }
       }
     }
@@ -1328,6 +1377,11 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// Both copy helpers write m0 (the LDS base of the copy) and say so in their
+// clobber lists, so that the compiler never assumes a value it put there
+// survives them; clang warns about any mention of m0 there, which is the point.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_offset,
                                                unsigned lds_address) {
   asm volatile(
@@ -1336,7 +1390,7 @@ __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_o
       "global_load_lds_dwordx4 %1, %2"
       :
       : "s"(lds_address), "v"(lane_offset), "s"(base)
-      : "memory");
+      : "memory", "m0");
 }
 
 // Same, with a full address per lane (planar layout: the 16 rows of a row block
@@ -1349,11 +1403,12 @@ __device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
       "global_load_lds_dwordx4 %1, off"
       :
       : "s"(lds_address), "v"(lane_address)
-      : "memory");
+      : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER,
-          int MS>
+          int MS, int XTM>
 __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma_dtl(
     const KernelArgs args) {
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
@@ -1375,6 +1430,20 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   constexpr int X_ROW_BLOCKS = X_BYTES / 1024;
   static_assert(ROW_BLOCKS % NW == 0, "row blocks must divide evenly over the waves");
   constexpr int LPW = ROW_BLOCKS / NW;              // loads per wave per K tile
+  // XTM 0: off; 1: exchanged MFMA roles (below); 2: also the early refill at the
+  // end of a C tile (see the pipeline)
+  constexpr bool XT = XTM != 0, EARLY = XTM == 2;
+  // XT: the X fragments feed the "B" side of the 16-row MFMA and tile i of a wave
+  // holds the columns x = 4 (lane % 16) + i of its 64, so that a lane ends up with
+  // 16 consecutive bytes of four C rows per register index and the C stores need no
+  // regrouping through LDS. For that, the rows of every 16-row block of X sit in
+  // LDS in the order [4 a + (i ^ a)] <- row 4 a + i, with their 16-byte chunks XORed
+  // with 3 (block & 1): fragment reads of rows 4 r + i are then free of bank
+  // conflicts (measured), and a copy instruction still moves the contiguous 1 KiB.
+  static_assert(!XT || (MS == 16 && KPM == 1 && TX == 4 && TY == 4 && !IL && WX == 64 &&
+                        X_ROW_BLOCKS % NW == 0 && NW % 2 == 0),
+                "exchanged roles: 16-row MFMA, 4 x 4 tiles per wave");
+  constexpr int X_LOADS = X_ROW_BLOCKS / NW;        // (XT) the first loads of a wave are X row blocks
   static_assert(SLOTS % KPI == 0 && SLOTS / KPI >= 2, "ring must hold at least two iterations");
   constexpr int LEAD = SLOTS / KPI - 1;             // iterations of prefetch distance
   static_assert((LEAD - 1) * KPI * LPW < 64, "vmcnt range");
@@ -1413,6 +1482,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   auto c_of = [&](int rb) {   // chunk this lane fetches for row block rb of an operand
     return (IL && MS == 32) ? ((lane % CPR) ^ (((rb & 1) << 2) | ((r >> 1) & 3))) : c;
   };
+  // (XT) row and chunk this lane fetches of an X row block (a wave's X row blocks
+  // all have the parity of the wave number)
+  const int xt_row = 4 * (lane >> 4) + (((lane >> 2) & 3) ^ (lane >> 4));
+  const int xt_chunk = (lane & 3) ^ (3 * (wave & 1));
+  const unsigned lane_off_x = XT ? xt_row * kTileRowBytes + xt_chunk * 16 : lane_off;
   {
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
@@ -1449,9 +1523,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes;
         } else {
           const unsigned total_rows = is_x ? args.nx : args.ny;
-          unsigned row = row0 + r;
+          const bool xt = XT && is_x;
+          unsigned row = row0 + (xt ? xt_row : r);
           row = row < total_rows ? row : total_rows - 1;   // likewise
-          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_stride + c_of(rb) * 16;
+          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_stride +
+                        (xt ? xt_chunk : c_of(rb)) * 16;
         }
       }
     }
@@ -1467,7 +1543,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
         const char *base = real ? src[i] + (size_t)load_kt * kTileBytes + tile_off[i] : g_zero_tile;
-        load_1k_to_lds(base, lane_off, lds_dst[i] + slot * SLOT_BYTES);
+        load_1k_to_lds(base, (XT && i < X_LOADS) ? lane_off_x : lane_off,
+                       lds_dst[i] + slot * SLOT_BYTES);
       }
     } else {
       // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
@@ -1475,7 +1552,8 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       for (int i = 0; i < LPW; ++i) {
         const int q = i * NW + wave;
         const int rb = (q < X_ROW_BLOCKS ? q : q - X_ROW_BLOCKS) % ((q < X_ROW_BLOCKS ? BX : BY) / RPB);
-        const bool inside = (load_kt * RB + c_of(rb) * 16 + 16 <= row_bytes);
+        const int chunk = (XT && q < X_ROW_BLOCKS) ? xt_chunk : c_of(rb);
+        const bool inside = (load_kt * RB + chunk * 16 + 16 <= row_bytes);
         const char *p = inside ? lane_src[i] + (size_t)load_kt * RB
                                : g_zero_tile + lane * 16;
         load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
@@ -1497,6 +1575,14 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
   const int x_frag_off = (wx * WX) * kTileRowBytes + frag_lane_off;
   const int y_frag_off = X_BYTES + (wy * WY) * kTileRowBytes + frag_lane_off;
+  int xo[4];   // X fragment of tile i (16-row MFMA)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r16 = lane & 15, g = lane >> 4;
+    xo[i] = XT ? (wx * WX + 4 * r16 + (i ^ (r16 & 3))) * kTileRowBytes +
+                     ((g ^ (3 * ((r16 >> 2) & 1))) * 16)
+               : x_frag_off + i * 16 * kTileRowBytes;
+  }
   // 32-row MFMA: row lane % 32, chunks lane / 32 and lane / 32 + 2 (any split
   // of K over the lanes is fine as long as X and Y use the same one)
   const int row32 = lane & 31, sw32 = (row32 >> 2) & 3;
@@ -1547,6 +1633,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   }
   unsigned slot = 0;                       // first slot of the current iteration
   const unsigned iters = k_tiles_padded / KPI;
+  // (EARLY) store instructions of the fast epilogue of one wave, and whether the
+  // previous tile's epilogue was that one
+  constexpr int kFastStores = 2 * TY * 4;
+  static_assert(!EARLY || (LEAD == 2 && KPI == 1 && kFastStores + LPW < 64), "early refill");
+  bool stores_in_flight = false;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
     typename AccType<MS>::type acc_re[TY][TX], acc_im[TY][TX];
 #pragma unroll
@@ -1558,13 +1649,24 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     for (unsigned it = 0; it < iters; ++it) {
-      if constexpr (KPI == 1) advance_copy();
+      // (EARLY) the first iteration of a C tile after the block's first issues no
+      // copies: the K tile it would fetch was requested before the previous
+      // tile's C stores
+      const bool no_refill = EARLY && it == 0 && vt != blockIdx.x;
+      if constexpr (KPI == 1) {
+        if (!no_refill) advance_copy();
+      }
       // After the first C tile, the K tiles of the first LEAD iterations were
       // already waited for before the previous epilogue (see below), so these
       // iterations only need the barrier; waiting on the counter here would
       // wait for the previous tile's C stores, which are younger than them.
       if (vt != blockIdx.x && it < (unsigned)LEAD) {
         asm volatile("s_barrier" ::: "memory");
+      } else if (EARLY && vt != blockIdx.x && it == (unsigned)LEAD && stores_in_flight) {
+        // the K tile of this iteration was requested before the C stores of the
+        // previous tile: they and this wave's copies of the next K tile may still be
+        // in flight (the counter retires in order)
+        wait_vmcnt_then_barrier<kFastStores + (LEAD - 1) * KPI * LPW>();
       } else {
         wait_vmcnt_then_barrier<(LEAD - 1) * KPI * LPW>();
       }
@@ -1605,7 +1707,11 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         } else if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
         } else if constexpr (KPM == 1 && TX == 4 && TY == 4) {
-          mma_step_ordered<DT, BX, BY>(tile[0], x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
+          if (no_refill) {
+            mma_step_ordered<DT, BX, BY, XT>(tile[0], xo, y_frag_off, acc_re, acc_im, [] {});
+          } else {
+            mma_step_ordered<DT, BX, BY, XT>(tile[0], xo, y_frag_off, acc_re, acc_im, refill_slots);
+          }
         } else {
           mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
         }
@@ -1622,7 +1728,30 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     const TileCoord tc = tile_coord(args, vt);
     const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
     bool staged = false;
-    if constexpr (MS == 16 && TOUT == kFloat32 && TX == 4 &&
+    if constexpr (EARLY) {
+      // The slot consumed last is free once every wave has left the K loop. The K
+      // tile that the next iteration would request is requested now, ahead of
+      // the C stores: the memory pipeline of the compute unit works in order, and
+      // a request behind 256 KiB of stores comes back after the iteration that
+      // needs it.
+      unsigned free_slot = slot + LEAD * KPI;
+      free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
+      asm volatile("s_barrier" ::: "memory");
+      advance_copy();
+      issue_copies(free_slot);
+    }
+    if constexpr (XT) {
+      // the accumulators already hold whole row segments
+      if (staged_ok && !args.c_interleaved && x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
+        store_wave_tile_rows<TOUT, TY>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+        stores_in_flight = true;
+      } else {
+        store_wave_tile<TOUT, TX, TY, kAcc16T>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
+        stores_in_flight = false;
+      }
+      staged = true;
+    }
+    if constexpr (!XT && MS == 16 && TOUT == kFloat32 && TX == 4 &&
                   NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
       if (staged_ok) {
         // The slot consumed last is free until the next refill, but other waves
@@ -1642,7 +1771,7 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
         }
       }
     }
-    if constexpr (MS == 16 && (TOUT == kFloat16 || TOUT == kBfloat16) && TX == 4 &&
+    if constexpr (!XT && MS == 16 && (TOUT == kFloat16 || TOUT == kBfloat16) && TX == 4 &&
                   NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
       if (staged_ok && !args.c_interleaved && args.nx % 8 == 0) {
         unsigned free_slot = slot + LEAD * KPI;
@@ -1732,7 +1861,7 @@ inline int compute_units() {
 }
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
-          int LOADER = kLoadTiled, int MS = 16>
+          int LOADER = kLoadTiled, int MS = 16, int XT = 0>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
   constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
@@ -1745,7 +1874,7 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS>;
+  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS, XT>;
   static std::atomic<bool> lds_allowed[kMaxDevices];
   if (hipError_t e = allow_lds(kernel, LDS_BYTES, lds_allowed)) return e;
   // persistent blocks: as many as are resident at once, each walking C tiles
@@ -1779,8 +1908,8 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     if constexpr (KPM == 1) {
       // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
       return p.variant == kOpt
-                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled>(p, stream)
-                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec>(p, stream);
+                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 2>(p, stream)
+                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, 2>(p, stream);
     } else {
       // fp8: the 32x32x64 MFMA takes one K tile per instruction, which lets the
       // same block shape and ring as for 16-bit input fit into LDS
@@ -1825,12 +1954,6 @@ hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
         return p.variant == kOpt
                    ? launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
                    : launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
-      }
-      break;
-    case kFp4Sign:
-      // the 1-bit GEMM's operands expanded to fp4 +-1, tiled; exact integer sums
-      if (p.type_out == kInt32 && p.variant == kOpt && !p.input_interleaved) {
-        return launch_dtl<kFp4Sign, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream);
       }
       break;
     default:

@@ -33,14 +33,25 @@ __device__ __forceinline__ unsigned bytes_of_nibble(unsigned b) {
   return ((b & 0xfu) * 0x00204081u) & 0x01010101u;
 }
 
-constexpr int kUnroll = 1;
+// 16 bytes at any address: one wide load (global memory takes any alignment on
+// this target; a load that straddles cache lines costs a little bandwidth).
+typedef uint4_t uint4_unaligned_t __attribute__((aligned(1)));
+
+template <bool ALIGNED> __device__ __forceinline__ uint4_t load16(const unsigned char *p) {
+  if constexpr (ALIGNED) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p));
+  } else {
+    return *reinterpret_cast<const uint4_unaligned_t *>(p);
+  }
+}
 
 // Planar: thread -> kPackPerThread times 16 input bytes, each half an output word;
 // lane pairs merge. A wave takes 64 * kPackPerThread consecutive groups, so every
 // load instruction reads 1 KiB contiguous and a thread has several in flight.
 // n16 = number of whole 16-byte groups that make whole words (2 per word).
 constexpr int kPackPerThread = 2;
-__global__ __launch_bounds__(256) void pack_planar_vec(const uint4_t *__restrict__ in,
+template <bool ALIGNED>
+__global__ __launch_bounds__(256) void pack_planar_vec(const unsigned char *__restrict__ in,
                                                        unsigned *__restrict__ out, size_t n16) {
   const size_t stride = (size_t)gridDim.x * 256 * kPackPerThread;
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -50,7 +61,7 @@ __global__ __launch_bounds__(256) void pack_planar_vec(const uint4_t *__restrict
 #pragma unroll
     for (int k = 0; k < kPackPerThread; ++k) {
       const size_t gi = base + k * 64 + lane;
-      v[k] = gi < n16 ? __builtin_nontemporal_load(in + gi) : uint4_t{0, 0, 0, 0};
+      v[k] = gi < n16 ? load16<ALIGNED>(in + gi * 16) : uint4_t{0, 0, 0, 0};
     }
 #pragma unroll
     for (int k = 0; k < kPackPerThread; ++k) {
@@ -63,24 +74,32 @@ __global__ __launch_bounds__(256) void pack_planar_vec(const uint4_t *__restrict
 }
 
 // Interleaved: thread -> 16 input bytes = 8 (re, im) pairs -> 8 real bits and
-// 8 imaginary bits; four lanes merge into one real and one imaginary word.
-// Requires N % 64 == 0 so that the imaginary half starts on a word boundary.
-__global__ __launch_bounds__(256) void pack_interleaved_vec(const uint4_t *__restrict__ in,
+// 8 imaginary bits; four lanes merge into one real and one imaginary word. As
+// in the planar kernel a wave takes 64 * kPackPerThread consecutive groups. The
+// input is `segments` buffers of seg16 groups each, one after the other, every one
+// packed on its own (all its real bits, then all its imaginary bits): one segment
+// is the reference's packing of a whole buffer, one per batch is what the
+// pipeline needs. A segment must hold a multiple of 64 samples, so that its
+// imaginary half starts on a word boundary and four lanes never straddle two.
+template <bool ALIGNED>
+__global__ __launch_bounds__(256) void pack_interleaved_vec(const unsigned char *__restrict__ in,
                                                             unsigned *__restrict__ out,
-                                                            size_t n16, size_t imag_word0) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-  for (; g < n16; g += stride * kUnroll) {
-    uint4_t v[kUnroll];
+                                                            size_t seg16, size_t segments) {
+  const size_t n16 = seg16 * segments;
+  const size_t stride = (size_t)gridDim.x * 256 * kPackPerThread;
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t seg_words = seg16 / 2;        // packed words of one segment
+  for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kPackPerThread; base < n16; base += stride) {
+    uint4_t v[kPackPerThread];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const size_t gi = g + u * stride;
-      v[u] = gi < n16 ? __builtin_nontemporal_load(in + gi) : uint4_t{0, 0, 0, 0};
+    for (int k = 0; k < kPackPerThread; ++k) {
+      const size_t gi = base + k * 64 + lane;
+      v[k] = gi < n16 ? load16<ALIGNED>(in + gi * 16) : uint4_t{0, 0, 0, 0};
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const size_t gi = g + u * stride;
-      const unsigned b = bits_of16(v[u]);  // bit 2p = re of pair p, bit 2p+1 = im
+    for (int k = 0; k < kPackPerThread; ++k) {
+      const size_t gi = base + k * 64 + lane;
+      const unsigned b = bits_of16(v[k]);  // bit 2p = re of pair p, bit 2p+1 = im
       // gather even bits into the low byte, odd bits into the second byte
       unsigned e = b & 0x5555u, o = (b >> 1) & 0x5555u;
       e = (e | (e >> 1)) & 0x3333u;
@@ -92,35 +111,43 @@ __global__ __launch_bounds__(256) void pack_interleaved_vec(const uint4_t *__res
       const unsigned mine = e | (o << 8);
       const unsigned l1 = __shfl_down(mine, 1), l2 = __shfl_down(mine, 2),
                      l3 = __shfl_down(mine, 3);
-      if ((threadIdx.x & 3) == 0 && gi < n16) {
+      if ((lane & 3) == 0 && gi < n16) {
         const unsigned re = (mine & 0xffu) | ((l1 & 0xffu) << 8) | ((l2 & 0xffu) << 16) |
                             ((l3 & 0xffu) << 24);
         const unsigned im = ((mine >> 8) & 0xffu) | (((l1 >> 8) & 0xffu) << 8) |
                             (((l2 >> 8) & 0xffu) << 16) | (((l3 >> 8) & 0xffu) << 24);
-        out[gi >> 2] = re;
-        out[imag_word0 + (gi >> 2)] = im;
+        const size_t seg = gi / seg16, local = gi % seg16;
+        unsigned *o_seg = out + seg * seg_words;
+        o_seg[local >> 2] = re;
+        o_seg[seg_words / 2 + (local >> 2)] = im;
       }
     }
   }
 }
 
-// Any N, any alignment: one thread per output word, byte loads.
+// Any N: one thread per output word, byte loads. For the end of a buffer that
+// is not whole words and for interleaved segments that are not multiples of 64
+// samples. Interleaved input is `segments` buffers of n samples each (see above);
+// word w then counts the words of all segments, ceil(n / 32) each.
 __global__ __launch_bounds__(256) void pack_scalar(const unsigned char *__restrict__ in,
                                                    unsigned *__restrict__ out, size_t n,
                                                    size_t first_word, size_t words,
                                                    int interleaved) {
   const size_t w = first_word + (size_t)blockIdx.x * 256 + threadIdx.x;
   if (w >= words) return;
+  const size_t seg_words = (n + 31) / 32;
+  const size_t seg = interleaved ? w / seg_words : 0, lw = interleaved ? w % seg_words : w;
+  const unsigned char *src = in + seg * n;
   unsigned v = 0;
   for (unsigned bit = 0; bit < 32; ++bit) {
-    const size_t t = w * 32 + bit;
+    const size_t t = lw * 32 + bit;
     if (t >= n) break;
     size_t idx = t;
     if (interleaved) {
       idx = 2 * t;
       if (idx >= n) idx -= n - 1;
     }
-    if (in[idx] != 0) v |= 1u << bit;
+    if (src[idx] != 0) v |= 1u << bit;
   }
   out[w] = v;
 }
@@ -129,8 +156,9 @@ __global__ __launch_bounds__(256) void pack_scalar(const unsigned char *__restri
 // in flight per thread (with one, the kernel waits on the latency of its reads),
 // and every store instruction of a wave writes 1 KiB contiguous.
 constexpr int kUnpackPerThread = 4;
+template <bool ALIGNED>
 __global__ __launch_bounds__(256) void unpack_vec(const unsigned *__restrict__ in,
-                                                  uint4_t *__restrict__ out, size_t n16) {
+                                                  unsigned char *__restrict__ out, size_t n16) {
   const size_t stride = (size_t)gridDim.x * 256 * kUnpackPerThread;
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kUnpackPerThread; base < n16;
@@ -146,9 +174,13 @@ __global__ __launch_bounds__(256) void unpack_vec(const unsigned *__restrict__ i
       const size_t g = base + k * 64 + lane;
       if (g < n16) {
         const unsigned h = (w[k] >> ((g & 1) * 16)) & 0xffffu;
-        __builtin_nontemporal_store(uint4_t{bytes_of_nibble(h), bytes_of_nibble(h >> 4),
-                                            bytes_of_nibble(h >> 8), bytes_of_nibble(h >> 12)},
-                                    out + g);
+        const uint4_t v = {bytes_of_nibble(h), bytes_of_nibble(h >> 4), bytes_of_nibble(h >> 8),
+                           bytes_of_nibble(h >> 12)};
+        if constexpr (ALIGNED) {
+          __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(out) + g);
+        } else {
+          *reinterpret_cast<uint4_unaligned_t *>(out + g * 16) = v;   // one wide store at any address
+        }
       }
     }
   }
@@ -177,23 +209,35 @@ unsigned grid_for(size_t items, size_t per_thread) {
 }  // namespace
 
 hipError_t launch_pack_bits(const unsigned char *in, unsigned *out, size_t n, int interleaved,
-                            hipStream_t stream) {
-  if (n == 0) return hipSuccess;
-  const size_t words = ceil_div(n, 32);
-  size_t vec_words = 0;  // words produced by the vector kernel
+                            hipStream_t stream, size_t segments) {
+  if (n == 0 || segments == 0) return hipSuccess;
+  if (!interleaved) {
+    n *= segments;   // planar packing is the same flat map whatever the batch structure
+    segments = 1;
+  }
+  const size_t seg_words = ceil_div(n, 32), words = seg_words * segments;
+  size_t vec_words = 0;  // words produced by the vector kernels
   const bool aligned = ((uintptr_t)in % 16 == 0);
-  if (aligned && !interleaved) {
+  if (!interleaved) {
     vec_words = n / 32;
     if (vec_words) {
       const size_t n16 = vec_words * 2;
-      hipLaunchKernelGGL(pack_planar_vec, dim3(grid_for(n16, kPackPerThread)), dim3(256), 0, stream,
-                         reinterpret_cast<const uint4_t *>(in), out, n16);
+      const dim3 grid(grid_for(n16, kPackPerThread));
+      if (aligned) {
+        hipLaunchKernelGGL(pack_planar_vec<true>, grid, dim3(256), 0, stream, in, out, n16);
+      } else {
+        hipLaunchKernelGGL(pack_planar_vec<false>, grid, dim3(256), 0, stream, in, out, n16);
+      }
     }
-  } else if (aligned && interleaved && n % 64 == 0) {
+  } else if (n % 64 == 0) {
     vec_words = words;
-    const size_t n16 = n / 16;
-    hipLaunchKernelGGL(pack_interleaved_vec, dim3(grid_for(n16, kUnroll)), dim3(256), 0, stream,
-                       reinterpret_cast<const uint4_t *>(in), out, n16, n / 64);
+    const size_t seg16 = n / 16;
+    const dim3 grid(grid_for(seg16 * segments, kPackPerThread));
+    if (aligned) {
+      hipLaunchKernelGGL(pack_interleaved_vec<true>, grid, dim3(256), 0, stream, in, out, seg16, segments);
+    } else {
+      hipLaunchKernelGGL(pack_interleaved_vec<false>, grid, dim3(256), 0, stream, in, out, seg16, segments);
+    }
   }
   if (vec_words < words) {
     const size_t rest = words - vec_words;
@@ -209,10 +253,14 @@ hipError_t launch_unpack_bits(const unsigned *in, unsigned char *out, size_t n,
                               hipStream_t stream) {
   if (n == 0) return hipSuccess;
   size_t done = 0;
-  if ((uintptr_t)out % 16 == 0 && n >= 16) {
+  if (n >= 16) {
     const size_t n16 = n / 16;
-    hipLaunchKernelGGL(unpack_vec, dim3(grid_for(n16, kUnpackPerThread)), dim3(256), 0, stream, in,
-                       reinterpret_cast<uint4_t *>(out), n16);
+    const dim3 grid(grid_for(n16, kUnpackPerThread));
+    if ((uintptr_t)out % 16 == 0) {
+      hipLaunchKernelGGL(unpack_vec<true>, grid, dim3(256), 0, stream, in, out, n16);
+    } else {
+      hipLaunchKernelGGL(unpack_vec<false>, grid, dim3(256), 0, stream, in, out, n16);
+    }
     done = n16 * 16;
   }
   if (done < n) {

@@ -38,6 +38,8 @@ struct Config {
 // name: type, block BX x BY, wave WX x WY, ring slots, MFMA rows
 static const std::vector<Config> kConfigs = {
     {"f16 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat16, kFloat32},
+    {"f16 256x128 w64x64 s3 m16 xt1", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 1>, kFloat16, kFloat32},
+    {"f16 256x128 w64x64 s3 m16 xt2", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 2>, kFloat16, kFloat32},
     {"f16 256x128 w64x64 s3 m32", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat16, kFloat32},
     {"f16 128x128 w64x64 s2 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"f16 128x128 w64x32 s4 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat16, kFloat32},
@@ -45,10 +47,10 @@ static const std::vector<Config> kConfigs = {
     {"f32 256x128 w64x64 s3 m16", launch_dtl<kFloat32, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat32, kFloat32},
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"fp8 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat8e4m3, kFloat32},
-    {"fp4 256x128 w64x64 s3 m32", launch_dtl<kFp4Sign, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFp4Sign, kInt32},
     {"int1 256x128 w64x64 s3 m32", launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kInt1, kInt32},
     // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
+    {"f16 planar 256x128 w64x64 s3 m16 xt2", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, 2>, kFloat16, kFloat32, kLoadPlanarVec},
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
     {"fp8 interleaved 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec, 16>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
@@ -58,8 +60,7 @@ static const std::vector<Config> kConfigs = {
 static double peak_of(int type) {
   switch (type) {
     case kFloat32: return 157.3;
-    case kInt1:
-    case kFp4Sign: return 10066.3;
+    case kInt1: return 10066.3;
     case kFloat8e4m3:
     case kFloat8e5m2: return 5033.2;
     default: return 2516.6;
@@ -76,8 +77,6 @@ static void fill(std::vector<unsigned short> &h, int type) {
       v = (unsigned short)(((r >> 8 & 1) << 15) | (e << (type == kFloat16 ? 10 : 7)) | (r >> 9 & (type == kFloat16 ? 0x3ff : 0x7f)));
     } else if (type == kInt1) {
       v = (unsigned short)(r >> 4);
-    } else if (type == kFp4Sign) {
-      v = (unsigned short)(0x2222 | ((r & 1) << 3) | ((r & 2) << 6) | ((r & 4) << 9) | ((r & 8) << 12));
     } else {
       v = (unsigned short)((r & 0x3f3f) | 0x2020);
     }

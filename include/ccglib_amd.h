@@ -67,6 +67,34 @@ CCGLIB_API const char *ccglib_last_error(void);
 CCGLIB_API const char *ccglib_version(void);
 
 /* ------------------------------------------------------------------------
+ * Process-wide options. No counterpart in the reference (whose only such
+ * channel is its JIT macros, src/mma/GEMM.cpp:140-214): they select code paths
+ * that produce the same results, for tests and for tuning. An option is read
+ * when an object is created (HOST_CHUNK_BYTES: at every host Run); setting
+ * one is not synchronised with other threads.
+ *   INT1_POPCOUNT    0 (default): the 1-bit GEMM runs on the matrix cores (fp4
+ *                    MFMA on +-1 values, exact); 1: XOR + population count on
+ *                    the vector ALUs, which is otherwise only the fallback.
+ *   BASIC_RETILE     1 (default): a basic-variant GEMM whose planar rows are not
+ *                    whole 16-byte chunks, or whose operands are not 16-byte
+ *                    aligned, owns a tiled copy of A and B and re-tiles into it
+ *                    at every Run; 0: it reads such rows in place through
+ *                    registers (several times slower, no extra memory).
+ *   HOST_CHUNK_BYTES 0 (default): ccglib_pipeline_run_host moves jobs of 8 MiB
+ *                    or more in chunks of whole batches of about 32 MiB; any
+ *                    other value: chunks of about that many bytes, whatever
+ *                    the size of the job.
+ * ---------------------------------------------------------------------- */
+enum {
+  CCGLIB_AMD_OPTION_INT1_POPCOUNT = 0,
+  CCGLIB_AMD_OPTION_BASIC_RETILE = 1,
+  CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES = 2,
+  CCGLIB_AMD_OPTION_COUNT = 3
+};
+CCGLIB_API int ccglib_amd_set_option(int option, size_t value);
+CCGLIB_API int ccglib_amd_get_option(int option, size_t *value);
+
+/* ------------------------------------------------------------------------
  * Complex GEMM  C[b] = alpha * A[b] * B[b]^T + beta * C[b]
  * Replaces ccglib::mma::GEMM: constructor include/ccglib/gemm/mma.h:42-49
  * (src/mma/GEMM.cpp:243-254), Run :50 (src/mma/GEMM.cpp:263-268),

@@ -27,3 +27,19 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def default_library_options():
+    """Every test starts from, and leaves behind, the library's default options
+    (ccglib_amd.set_option), so that a test which selects a code path cannot leak
+    its choice into the next one."""
+    try:
+        import ccglib_amd as cc
+        defaults = {o: cc.get_option(o) for o in cc.Option}
+    except (RuntimeError, OSError):
+        yield          # library not built: tests that need it fail on their own
+        return
+    yield
+    for o, v in defaults.items():
+        cc.set_option(o, v)

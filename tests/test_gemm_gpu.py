@@ -144,12 +144,12 @@ def test_opt(tin, tout, M, N, K, c_order, c_axis):
     float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=True, seed=5)
 
 
-def basic_variant(variant, monkeypatch):
+def basic_variant(variant):
     """The basic variant copies operands with ragged rows (K·size not a multiple of 16
     bytes) into the tiled layout first; "basic_no_retile" switches that off, which
     leaves the kernel that loads ragged rows itself."""
     if variant == "basic_no_retile":
-        monkeypatch.setenv("CCGLIB_AMD_BASIC_RETILE", "0")
+        cc.set_option(cc.Option.basic_retile, 0)
         return cc.Variant.basic
     return variant
 
@@ -157,16 +157,16 @@ def basic_variant(variant, monkeypatch):
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000),
                                    (257, 129, 72), (130, 2, 2049)])
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt, "basic_no_retile"])
-def test_odd_shapes_fp16(M, N, K, variant, monkeypatch):
-    variant = basic_variant(variant, monkeypatch)
+def test_odd_shapes_fp16(M, N, K, variant):
+    variant = basic_variant(variant)
     float_case(2, M, N, K, VT.float16, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (17, 5, 3), (129, 131, 33), (64, 300, 1000), (257, 129, 72)])
 @pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt, "basic_no_retile"])
-def test_odd_shapes_fp32(M, N, K, variant, monkeypatch):
+def test_odd_shapes_fp32(M, N, K, variant):
     # K not a multiple of the 16 values of a tile row, rows that are not whole 16-byte chunks
-    variant = basic_variant(variant, monkeypatch)
+    variant = basic_variant(variant)
     float_case(2, M, N, K, VT.float32, VT.float32, variant, PLANAR, ROW, seed=M + N + K)
 
 
@@ -215,11 +215,10 @@ def test_fp32_alpha_beta_and_many_tiles():
 
 @pytest.mark.parametrize("tin", [VT.float8e4m3, VT.float8e5m2])
 @pytest.mark.parametrize("K", [1, 63, 64, 65, 128, 192, 200])
-def test_fp8_k_tails(tin, K, monkeypatch):
+def test_fp8_k_tails(tin, K):
     # an MFMA consumes two 64-value K tiles; odd tile counts and ragged tails
     float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=K)
-    with monkeypatch.context() as m:
-        m.setenv("CCGLIB_AMD_BASIC_RETILE", "0")
+    with cc.option(cc.Option.basic_retile, 0):
         float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=K)
     float_case(2, 70, 50, K, tin, VT.float32, cc.Variant.opt, PLANAR, COL, seed=K + 1)
 
@@ -281,24 +280,16 @@ def test_batches_are_independent():
 
 # ---- 1-bit ------------------------------------------------------------------------------
 
-@pytest.fixture(params=["mfma", "expand", "expand_grouped", "popcount"])
-def int1_kernel(request, monkeypatch):
-    """The 1-bit GEMM has three implementations behind one entry point: the fp4 MFMA
+@pytest.fixture(params=["mfma", "popcount"])
+def int1_kernel(request):
+    """The 1-bit GEMM has two implementations behind one entry point: the fp4 MFMA
     kernel that expands the packed words in registers (default, where the layout
-    allows it: tiled operands, or planar rows of whole 16-byte chunks), the same
-    MFMA on an expanded copy of the operands ("expand"; "grouped" = a workspace cap
-    that forces several passes over groups of batches) and XOR + popcount on the
-    vector ALUs (used when K is too large for exact fp32 sums or the workspace
-    cannot be had). The choice is read from the environment when the GEMM object is
+    allows it: tiled operands, planar rows of whole 16-byte chunks, other planar
+    rows after re-tiling) and XOR + popcount on the vector ALUs (the fallback, which
+    the option selects for everything). The option is read when the GEMM object is
     created."""
-    monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
-    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
     if request.param == "popcount":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
-    elif request.param.startswith("expand"):
-        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
-        if request.param == "expand_grouped":
-            monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+        cc.set_option(cc.Option.int1_popcount, 1)
     return request.param
 
 
@@ -424,7 +415,7 @@ def test_int1_several_c_tiles_per_block(variant, K):
 def test_int1_k_in_pieces(variant, K, int1_kernel):
     # two and three pieces, the last one a partial tile; alpha and beta applied once
     if variant == cc.Variant.basic and K % 128:
-        K -= K % 128       # planar rows of whole 16-byte chunks, or the popcount kernel runs
+        K -= K % 128       # planar rows of whole 16-byte chunks (no tiled copy of 2 x 8 MiB rows)
     int1_case(2, 40, 24, K, variant, c_order=COL, alpha=2 - 1j, beta=1 + 3j, seed=K % 1000)
 
 

@@ -108,6 +108,52 @@ def test_matches_complex128_matmul_exactly_on_small_integers(vtype, c_order):
     assert np.array_equal(c[:, 0], want.real) and np.array_equal(c[:, 1], want.imag)
 
 
+def _enc_any(vals, vtype):
+    """Small integers / powers of two into the storage type, fp8 included."""
+    v = np.asarray(vals, dtype=np.float32)
+    if vtype == orc.FLOAT8E4M3:
+        return torch.from_numpy(v).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    if vtype == orc.FLOAT8E5M2:
+        return torch.from_numpy(v).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    return enc(v, vtype)
+
+
+@pytest.mark.parametrize("vtype", [orc.FLOAT16, orc.BFLOAT16, orc.FLOAT32, orc.FLOAT8E4M3,
+                                   orc.FLOAT8E5M2])
+@pytest.mark.parametrize("c_order", [orc.ROW_MAJOR, orc.COL_MAJOR])
+def test_float64_yardstick_matches_complex128_matmul_exactly(vtype, c_order):
+    # The float64 product that the Frobenius criterion is measured against: on
+    # exactly representable small integers every product and partial sum is
+    # exact in double, so it must equal numpy's complex128 product bit for bit
+    # (a dropped term, wrong sign, conjugate or transposed operand fails here).
+    rng = np.random.default_rng(23)
+    B, M, N, K = 2, 7, 5, 19
+    # every value in [-4, 4] is exact in all five input types (e5m2 has two mantissa bits)
+    av = rng.integers(-4, 5, size=(B, 2, M, K))
+    bv = rng.integers(-4, 5, size=(B, 2, N, K))
+    A = av[:, 0] + 1j * av[:, 1]
+    Bm = bv[:, 0] + 1j * bv[:, 1]
+    want = np.einsum("bmk,bnk->bmn", A, Bm)
+    if c_order == orc.COL_MAJOR:
+        want = want.transpose(0, 2, 1)
+    a, b = _enc_any(av.reshape(-1), vtype), _enc_any(bv.reshape(-1), vtype)
+    assert np.array_equal(orc.to_float(a, vtype) if vtype != orc.FLOAT32 else a,
+                          av.reshape(-1).astype(np.float32))            # the encoding is exact
+    c = orc.gemm_float64(a, b, M, N, K, vtype, c_order)
+    assert c.dtype == np.float64
+    assert np.array_equal(c[:, 0], want.real) and np.array_equal(c[:, 1], want.imag)
+
+
+def test_float64_yardstick_keeps_what_float32_loses():
+    # 2^13 * 2^13 + 1 - 2^26 = 1 in double, 0 in float: the yardstick accumulates in
+    # double (and so can tell a float32 rounding error from a wrong result)
+    a = enc([8192.0, 1.0, -8192.0, 0, 0, 0], orc.FLOAT16)   # re[3], im[3]
+    b = enc([8192.0, 1.0, 8192.0, 0, 0, 0], orc.FLOAT16)
+    c64 = orc.gemm_float64(a, b, 1, 1, 3, orc.FLOAT16)
+    c32 = orc.gemm(a, b, 1, 1, 3, orc.FLOAT16)
+    assert c64[0, 0, 0, 0] == 1.0 and c32[0, 0, 0, 0] == 0.0
+
+
 def test_beta_zero_never_reads_c():
     a = enc(np.ones(2 * 2 * 4), orc.FLOAT16)
     c_in = np.full(2 * 2 * 2, np.nan, dtype=np.float32)

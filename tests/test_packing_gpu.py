@@ -95,6 +95,31 @@ def test_unaligned_buffers():
     assert np.array_equal(to_host(d_bytes, np.uint8)[5:5 + N], x[3:])
 
 
+@pytest.mark.parametrize("offset", [1, 4, 15])
+@pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
+def test_unaligned_large_buffers(offset, axis):
+    # buffers at odd addresses take the same wide-access kernels (one 16-byte access at any
+    # address), also beyond one grid of blocks' worth of data
+    rng = np.random.default_rng(offset)
+    N = (1 << 21) + 64 + (13 if axis == PLANAR else 0)
+    x = rng.integers(0, 2, N + offset, dtype=np.uint8)
+    d_in = to_device(x)
+    words = (N + 31) // 32
+    d_out = to_device(np.full(words + 2, 0xDEADBEEF, dtype=np.uint32))
+    cc.Packing(N, cc.Direction.forward, 0, stream(), axis).Run(d_in.data_ptr() + offset, d_out.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_out, np.uint32)
+    assert np.array_equal(got[:words], orc.pack_bits(x[offset:].copy(), int(axis)))
+    assert np.all(got[words:] == 0xDEADBEEF)
+    if axis == PLANAR:
+        d_bytes = to_device(np.full(N + 32, 9, dtype=np.uint8))
+        cc.Packing(N, cc.Direction.backward, 0, stream()).Run(d_out.data_ptr(), d_bytes.data_ptr() + offset)
+        torch.cuda.synchronize()
+        back = to_host(d_bytes, np.uint8)
+        assert np.array_equal(back[offset:offset + N], x[offset:])
+        assert np.all(back[:offset] == 9) and np.all(back[offset + N:] == 9)
+
+
 def test_host_input():
     rng = np.random.default_rng(6)
     N = 2048

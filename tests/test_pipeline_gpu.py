@@ -1,6 +1,5 @@
 """GPU parity tests of the pipeline wrapper (pack -> transpose -> GEMM) against the
 CPU oracle; cases follow the reference's test/pipeline/pipeline.cpp."""
-import functools
 
 import numpy as np
 import pytest
@@ -102,22 +101,15 @@ def test_pipeline_int1(variant):
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
-@pytest.mark.parametrize("mode", ["direct", "expand", "popcount", "capped_workspace"])
+@pytest.mark.parametrize("mode", ["direct", "popcount"])
 @pytest.mark.parametrize("M,N,K,c_order", [(130, 70, 992, ROW), (64, 200, 96, COL), (20, 30, 32, ROW),
                                            (256, 128, 2048, COL)])
-def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
+def test_pipeline_int1_shapes(mode, M, N, K, c_order):
     # Planar one-byte-per-sample input is packed straight into the tiled 1-bit layout
-    # in the GEMM's workspace ("direct") or expanded into fp4 values there ("expand");
-    # without a (whole) workspace the pipeline packs and transposes as the reference
-    # does. Any non-zero byte is a 1 bit.
-    monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
-    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
+    # in the GEMM's workspace ("direct"); with the vector-ALU kernel selected the
+    # pipeline packs and transposes as the reference does. Any non-zero byte is a 1 bit.
     if mode == "popcount":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
-    elif mode == "expand":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
-    elif mode == "capped_workspace":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
+        cc.set_option(cc.Option.int1_popcount, 1)
     B = 3
     rng = np.random.default_rng(M + K)
     a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
@@ -139,15 +131,12 @@ def test_pipeline_int1_shapes(mode, M, N, K, c_order, monkeypatch):
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
-@pytest.mark.parametrize("mode", ["direct", "expand"])
-def test_pipeline_int1_unaligned_input(mode, monkeypatch):
+@pytest.mark.parametrize("mode", ["direct", "popcount"])
+def test_pipeline_int1_unaligned_input(mode):
     # input buffers that start at an odd address: the kernels that read the bytes 16 at a
-    # time fall back to byte loads
-    monkeypatch.delenv("CCGLIB_AMD_INT1_WORKSPACE_MB", raising=False)
-    if mode == "expand":
-        monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
-    else:
-        monkeypatch.delenv("CCGLIB_AMD_INT1_KERNEL", raising=False)
+    # time use unaligned loads or fall back to byte loads
+    if mode == "popcount":
+        cc.set_option(cc.Option.int1_popcount, 1)
     B, M, N, K = 2, 150, 140, 1056
     rng = np.random.default_rng(5)
     a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
@@ -161,51 +150,6 @@ def test_pipeline_int1_unaligned_input(mode, monkeypatch):
     torch.cuda.synchronize()
     want = orc.gemm(pack_rows(a_bits, B, M, K), pack_rows(b_bits, B, N, K), M, N, K, orc.INT1, orc.INT32)
     assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
-
-
-@functools.lru_cache(maxsize=1)
-def _grouped_int1_case(B, M, N, K):
-    """Two sets of random 1-bit operands (one byte per sample) and the oracle's C for each."""
-    rng = np.random.default_rng(77)
-    bits = [[rng.integers(0, 2, B * 2 * rows * K, dtype=np.uint8) for rows in (M, N)] for _ in range(2)]
-    wants = [orc.gemm(orc.pack_bits(a), orc.pack_bits(b), M, N, K, orc.INT1, orc.INT32) for a, b in bits]
-    return bits, wants
-
-
-@pytest.mark.parametrize("overlap", [True, False])
-@pytest.mark.parametrize("what", ["pipeline", "gemm_opt", "gemm_basic"])
-def test_int1_expansion_in_groups(what, overlap, monkeypatch):
-    """Enough batches and C tiles (16 x 32 tiles of 256 x 128) for the 1-bit GEMM to expand and
-    multiply in two groups of 8 batches, the expansion on a second stream (or, with
-    CCGLIB_AMD_INT1_OVERLAP=0, everything on the caller's stream). Two Runs in a row with
-    different input: the second call's expansion must not overtake the first call's GEMMs."""
-    # (the MFMA kernel on an fp4 copy of the operands; by default the packed words
-    # are multiplied as they are and nothing is expanded)
-    monkeypatch.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
-    if not overlap:
-        monkeypatch.setenv("CCGLIB_AMD_INT1_OVERLAP", "0")
-    B, M, N, K = 16, 1024, 1024, 256
-    bits, wants = _grouped_int1_case(B, M, N, K)
-    d_c = [to_device(np.zeros(B * 2 * M * N, dtype=np.int32)) for _ in range(2)]
-    if what == "pipeline":
-        obj = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
-                          cc.Variant.opt)
-        d_in = [[to_device(x) for x in pair] for pair in bits]
-    else:
-        variant = cc.Variant.opt if what == "gemm_opt" else cc.Variant.basic
-        obj = cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(VT.int1, VT.int32), variant)
-        packed = [[orc.pack_bits(x) for x in pair] for pair in bits]
-        if what == "gemm_opt":
-            from gpu_util import transpose_operand
-            d_in = [[transpose_operand(x, B, rows, K, VT.int1) for x, rows in zip(pair, (M, N))]
-                    for pair in packed]
-        else:
-            d_in = [[to_device(x) for x in pair] for pair in packed]
-    for i in range(2):
-        obj.Run(d_in[i][0].data_ptr(), d_in[i][1].data_ptr(), d_c[i].data_ptr())
-    torch.cuda.synchronize()
-    for i in range(2):
-        assert np.array_equal(to_host(d_c[i], np.int32).reshape(wants[i].shape), wants[i])
 
 
 def pack_rows(bits, B, rows, K):
@@ -233,12 +177,12 @@ def _host_buffer(a, pinned):
     (6, 256, 1024, 128, PLANAR, 0.5 - 0.25j, None),      # default size: 2 chunks of 3 batches
     (8, 256, 512, 256, INTERLEAVED, 0, 1 << 20),         # 8 chunks of 1: every lane used again
     (7, 200, 1000, 104, INTERLEAVED, 0, 5 << 20)])       # 2.1 MB a batch: chunks of 2, 2, 2 and 1
-def test_pipeline_host_run_in_chunks(pinned, B, M, N, K, axis, beta, chunk_bytes, monkeypatch):
+def test_pipeline_host_run_in_chunks(pinned, B, M, N, K, axis, beta, chunk_bytes):
     """Host-pointer Run of a problem that takes the batch-chunked path over several
     streams: equal, bit for bit, to the device Run of the same object, and within the
     float bounds of the oracle."""
     if chunk_bytes:
-        monkeypatch.setenv("CCGLIB_AMD_HOST_CHUNK_BYTES", str(chunk_bytes))
+        cc.set_option(cc.Option.host_chunk_bytes, chunk_bytes)
     alpha = 1.0 if beta == 0 else 2 - 1j
     rng = np.random.default_rng(11)
     qa = quantize(rng.uniform(-2, 2, B * 2 * M * K), VT.float16)
@@ -265,10 +209,19 @@ def test_pipeline_host_run_in_chunks(pinned, B, M, N, K, axis, beta, chunk_bytes
     check_float(hc.reshape(want.shape), want, np.stack([w.real, w.imag], 1), VT.float16, VT.float32)
 
 
+def pack_per_batch(bits, B, axis):
+    """The oracle's packing of one-byte-per-sample input, batch by batch: for interleaved
+    input ([rows][K][2] per batch) all real bits of a batch, then all its imaginary bits
+    (kernels/packing_kernel.cu:15-22 applied to one batch), which is the planar layout
+    [B][2][rows][K / 32] that the 1-bit GEMM reads."""
+    per = bits.reshape(B, -1)
+    return np.concatenate([orc.pack_bits(np.ascontiguousarray(x), int(axis)) for x in per])
+
+
 @pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
 def test_pipeline_int1_host_run(axis):
-    """1-bit host Run: planar input goes through the chunked path (2 chunks of 2 batches:
-    13 MiB in all), interleaved input (packed over the whole buffer) in one piece."""
+    """1-bit host Run through the chunked path (2 chunks of 2 batches: 13 MiB in all), planar
+    and interleaved input: the oracle's integers, from the device Run and from the host Run."""
     B, M, N, K = 4, 128, 256, 4096
     rng = np.random.default_rng(12)
     a_bits = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8)
@@ -281,11 +234,59 @@ def test_pipeline_int1_host_run(axis):
     torch.cuda.synchronize()
     got = c.copy()
     p.RunHost(a_bits.ctypes.data, b_bits.ctypes.data, got.ctypes.data)
-    assert np.array_equal(got, to_host(d_c, np.int32))
-    if axis == PLANAR:
-        want = orc.gemm(orc.pack_bits(a_bits), orc.pack_bits(b_bits), M, N, K, orc.INT1, orc.INT32,
-                        orc.ROW_MAJOR, 1.0, 1.0, c)
-        assert np.array_equal(got.reshape(want.shape), want)
+    want = orc.gemm(pack_per_batch(a_bits, B, axis), pack_per_batch(b_bits, B, axis), M, N, K,
+                    orc.INT1, orc.INT32, orc.ROW_MAJOR, 1.0, 1.0, c)
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+    assert np.array_equal(got.reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("kernel", ["mfma", "popcount"])
+@pytest.mark.parametrize("variant", [cc.Variant.opt, cc.Variant.basic])
+@pytest.mark.parametrize("B,M,N,K,c_order", [(1, 64, 48, 256, ROW), (1, 130, 70, 992, COL),
+                                             (3, 64, 200, 96, ROW), (5, 20, 30, 1024, COL)])
+def test_pipeline_int1_interleaved_input(kernel, variant, B, M, N, K, c_order):
+    """1-bit pipeline with interleaved input (one byte per sample, [B][rows][K][2]): for one
+    batch the reference's flat packing (kernels/packing_kernel.cu:15-22) is the planar
+    layout; for several batches every batch is packed on its own. Device Run and host Run
+    against the oracle's GEMM of the oracle's packing, bit for bit; any non-zero byte is a 1."""
+    if kernel == "popcount":
+        cc.set_option(cc.Option.int1_popcount, 1)
+    rng = np.random.default_rng(B * 1000 + K)
+    a_bits = rng.integers(0, 2, B * M * K * 2, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * N * K * 2, dtype=np.uint8)
+    a_in = a_bits * rng.integers(1, 256, a_bits.size, dtype=np.uint8)
+    b_in = b_bits * rng.integers(1, 256, b_bits.size, dtype=np.uint8)
+    alpha, beta = 2 - 1j, -1 + 1j
+    c_in = rng.integers(-1000, 1000, B * 2 * M * N).astype(np.int32)
+    want = orc.gemm(pack_per_batch(a_bits, B, INTERLEAVED), pack_per_batch(b_bits, B, INTERLEAVED),
+                    M, N, K, orc.INT1, orc.INT32, int(c_order), alpha, beta, c_in)
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, c_order, VT.int1,
+                    VT.int32, variant, alpha, beta)
+    d_a, d_b, d_c = to_device(a_in), to_device(b_in), to_device(c_in)
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
+    got = c_in.copy()
+    p.RunHost(a_in.ctypes.data, b_in.ctypes.data, got.ctypes.data)
+    assert np.array_equal(got.reshape(want.shape), want)
+
+
+def test_pipeline_int1_interleaved_input_unaligned():
+    # interleaved bytes at an odd address: the packing kernel's wide loads take any address
+    B, M, N, K = 2, 96, 64, 512
+    rng = np.random.default_rng(8)
+    a_bits = rng.integers(0, 2, B * M * K * 2, dtype=np.uint8)
+    b_bits = rng.integers(0, 2, B * N * K * 2, dtype=np.uint8)
+    want = orc.gemm(pack_per_batch(a_bits, B, INTERLEAVED), pack_per_batch(b_bits, B, INTERLEAVED),
+                    M, N, K, orc.INT1, orc.INT32, c_in=np.zeros(B * 2 * M * N, np.int32))
+    d_a = to_device(np.concatenate([np.zeros(1, np.uint8), a_bits]))
+    d_b = to_device(np.concatenate([np.zeros(5, np.uint8), b_bits]))
+    d_c = to_device(np.zeros(B * 2 * M * N, np.int32))
+    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, VT.int1, VT.int32,
+                    cc.Variant.opt)
+    p.Run(d_a.data_ptr() + 1, d_b.data_ptr() + 5, d_c.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host(d_c, np.int32).reshape(want.shape), want)
 
 
 @pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.float16, VT.float16),

@@ -90,10 +90,9 @@ def _pack_rows(bits, B, rows, K):
 
 
 @pytest.mark.parametrize("seed", [21, 22])
-def test_random_int1_cases(seed, monkeypatch):
+def test_random_int1_cases(seed):
     """1-bit GEMM and pipeline, bit-exact: both variants, ragged shapes, integer alpha / beta,
-    and the switches that select the popcount kernel, a capped workspace (several passes) or
-    a single stream."""
+    and the option that selects the popcount kernel."""
     rng = np.random.default_rng(seed)
     for case in range(40):
         B = int(rng.integers(1, 6))
@@ -107,18 +106,8 @@ def test_random_int1_cases(seed, monkeypatch):
         c_order = ROW if rng.integers(2) else COL
         alpha = complex(int(rng.integers(-3, 4)), int(rng.integers(-3, 4)))
         beta = complex(int(rng.integers(-2, 3)), int(rng.integers(-2, 3))) if rng.integers(2) else 0j
-        switch = int(rng.integers(6))
-        with monkeypatch.context() as env:
-            for name in ("CCGLIB_AMD_INT1_KERNEL", "CCGLIB_AMD_INT1_WORKSPACE_MB", "CCGLIB_AMD_INT1_OVERLAP"):
-                env.delenv(name, raising=False)
-            if switch == 1:
-                env.setenv("CCGLIB_AMD_INT1_KERNEL", "popcount")
-            elif switch >= 2:
-                env.setenv("CCGLIB_AMD_INT1_KERNEL", "expand")
-                if switch == 3:
-                    env.setenv("CCGLIB_AMD_INT1_WORKSPACE_MB", "1")
-                elif switch == 4:
-                    env.setenv("CCGLIB_AMD_INT1_OVERLAP", "0")
+        switch = int(rng.integers(3))   # 1: the vector-ALU kernel; else the default (MFMA)
+        with cc.option(cc.Option.int1_popcount, 1 if switch == 1 else 0):
             print("seed %d case %d: B=%d M=%d N=%d K=%d way %d C %s alpha=%s beta=%s switch %d" % (
                 seed, case, B, M, N, K, way, "row" if c_order == ROW else "col", alpha, beta, switch),
                 flush=True)
