@@ -223,3 +223,18 @@ class Pipeline(_Handle):
         _capi.check(_capi.load().ccglib_pipeline_run_host(self._h, _ptr(h_a), _ptr(h_b),
                                                          _ptr(h_c)))
 
+
+STATIC_SCRATCH_BYTES = 32 << 20   # CCGLIB_AMD_STATIC_SCRATCH_BYTES in include/ccglib_amd.h
+
+
+def pipeline_run_static(B, M, N, K, device, stream, input_complex_axis_location,
+                        output_complex_axis_location, a_mem_order, b_mem_order, c_mem_order,
+                        input_precision, output_precision, variant, alpha, beta, d_a, d_b, d_c):
+    """The pipeline as one stateless call that allocates nothing: its scratch is a static
+    device array (ccglib_pipeline_run_static; no counterpart in the reference)."""
+    alpha, beta = complex(alpha), complex(beta)
+    _capi.check(_capi.load().ccglib_pipeline_run_static(
+        B, M, N, K, device, _ptr(stream), int(input_complex_axis_location),
+        int(output_complex_axis_location), int(a_mem_order), int(b_mem_order), int(c_mem_order),
+        int(input_precision), int(output_precision), int(variant), alpha.real, alpha.imag,
+        beta.real, beta.imag, _ptr(d_a), _ptr(d_b), _ptr(d_c)))

@@ -34,6 +34,8 @@ SIGNATURES = {
     "ccglib_pipeline_run": (_i, [_vp, _vp, _vp, _vp]),
     "ccglib_pipeline_run_host": (_i, [_vp, _vp, _vp, _vp]),
     "ccglib_pipeline_destroy": (_i, [_vp]),
+    "ccglib_pipeline_run_static": (_i, [_sz, _sz, _sz, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
+                                        _f, _f, _f, _f, _vp, _vp, _vp]),
 }
 
 _lib = None

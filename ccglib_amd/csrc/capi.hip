@@ -1056,3 +1056,151 @@ int ccglib_pipeline_run_host(ccglib_pipeline_t p, const void *h_a, const void *h
 }
 
 }  // extern "C"
+
+/* ---------------------- Pipeline without allocations --------------------- */
+
+namespace {
+
+// Scratch of the stateless pipeline call: the tiled (and, for 1-bit
+// interleaved input, packed) copies of A and B that a pipeline object keeps in
+// memory it allocates. One array per GPU, held from the moment the library's
+// code is loaded there until the process ends; every call on that GPU uses it.
+constexpr size_t kStaticScratchBytes = CCGLIB_AMD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on each GPU. In host code the array's name is only
+// a handle for hipGetSymbolAddress, never an address a kernel could use.
+constexpr int kMaxScratchDevices = 64;
+unsigned char *g_scratch_ptr[kMaxScratchDevices] = {};
+std::atomic<bool> g_scratch_ready[kMaxScratchDevices];
+
+// First call on a device: checks the device and looks up its copy of the array
+// (with that device current).
+int static_scratch(int device, unsigned char **ptr) {
+  if (device < 0 || device >= kMaxScratchDevices) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "device ordinal %d out of range", device);
+  }
+  if (!g_scratch_ready[device].load(std::memory_order_acquire)) {
+    if (int rc = check_device(device)) return rc;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail_hip(e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[device] = static_cast<unsigned char *>(p);
+    g_scratch_ready[device].store(true, std::memory_order_release);
+  }
+  *ptr = g_scratch_ptr[device];
+  return CCGLIB_OK;
+}
+
+size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+
+extern "C" {
+
+int ccglib_pipeline_run_static(size_t B, size_t M, size_t N, size_t K, int device, void *stream,
+                               int input_complex_axis_location,
+                               int output_complex_axis_location, int a_mem_order,
+                               int b_mem_order, int c_mem_order, int input_type, int output_type,
+                               int variant, float alpha_re, float alpha_im, float beta_re,
+                               float beta_im, const void *d_a, const void *d_b, void *d_c) {
+  if (!is_enum01(input_complex_axis_location)) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "enum argument out of range");
+  }
+  if (int rc = validate_gemm(B, M, N, K, input_type, output_type, variant,
+                             output_complex_axis_location, c_mem_order, a_mem_order,
+                             b_mem_order)) {
+    return rc;
+  }
+  if (B == 0 || M == 0 || N == 0) return CCGLIB_OK;
+  if (K == 0) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "K = 0 has no tiled layout");
+  if (!d_a || !d_b || !d_c) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  const bool int1 = (input_type == kInt1);
+  if (int1 && K % 32 != 0) {
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "1-bit input needs K to be a multiple of 32 here (got %zu)", K);
+  }
+  DeviceGuard guard(device);
+  HIP_TRY(guard.status());
+  unsigned char *ws = nullptr;
+  if (int rc = static_scratch(device, &ws)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  // The GEMM always reads tiled copies here (what the opt variant reads; for the
+  // basic variant the same numbers, as the kernels only differ in their loaders).
+  ccglib_gemm g;
+  init_gemm(&g, B, M, N, K, device, stream, input_type, output_type, kOpt,
+            output_complex_axis_location, c_mem_order, alpha_re, alpha_im, beta_re, beta_im);
+  size_t tiled_a = 0, tiled_b = 0;
+  tiled_bytes(&g, &tiled_a, &tiled_b);
+  const bool pack_first = int1 && input_complex_axis_location == kInterleaved;
+  const size_t packed_a = pack_first ? round_up_256(B * 2 * M * K / 8) : 0;
+  const size_t packed_b = pack_first ? round_up_256(B * 2 * N * K / 8) : 0;
+  const size_t need = round_up_256(tiled_a) + round_up_256(tiled_b) + packed_a + packed_b;
+  if (need > kStaticScratchBytes) {
+    return fail(CCGLIB_ERROR_UNSUPPORTED,
+                "ccglib_pipeline_run_static: the tiled copies of A and B take %zu bytes, the "
+                "static scratch holds %zu; use a pipeline object for this size", need,
+                kStaticScratchBytes);
+  }
+  unsigned char *ws_a = ws, *ws_b = ws + round_up_256(tiled_a);
+  unsigned char *ws_pa = ws_b + round_up_256(tiled_b), *ws_pb = ws_pa + packed_a;
+
+  if (int1 && !pack_first) {
+    // one byte per sample, planar: packed straight into 1-bit tiles, then multiplied
+    g.workspace = ws;
+    g.workspace_bytes = tiled_a + tiled_b;
+    GemmParams q;
+    fill_gemm_params(&g, d_a, d_b, d_c, &q);
+    q.int1_direct = 1;
+    if (!gemm_int1_can_take_bytes(q)) {
+      return fail(CCGLIB_ERROR_UNSUPPORTED, "ccglib_pipeline_run_static: 1-bit problem out of range");
+    }
+    // (the packing kernel writes A's tiles and B's tiles back to back)
+    const hipError_t e = launch_gemm_int1_from_bytes(q, s);
+    if (e != hipSuccess) return fail_hip(e, "1-bit pipeline launch");
+    return CCGLIB_OK;
+  }
+
+  const void *src_a = d_a, *src_b = d_b;
+  int axis = input_complex_axis_location;
+  if (pack_first) {
+    // every batch packed on its own: real bits, then imaginary bits (planar)
+    if ((M * K) % 32 != 0 || (N * K) % 32 != 0) {
+      return fail(CCGLIB_ERROR_UNSUPPORTED, "1-bit interleaved input needs M*K and N*K to be multiples of 32");
+    }
+    hipError_t e = launch_pack_bits(static_cast<const unsigned char *>(d_a),
+                                    reinterpret_cast<unsigned *>(ws_pa), 2 * M * K, 1, s, B);
+    if (e == hipSuccess) {
+      e = launch_pack_bits(static_cast<const unsigned char *>(d_b),
+                           reinterpret_cast<unsigned *>(ws_pb), 2 * N * K, 1, s, B);
+    }
+    if (e != hipSuccess) return fail_hip(e, "packing kernel launch");
+    src_a = ws_pa;
+    src_b = ws_pb;
+    axis = kPlanar;
+  }
+  TransposeParams t;
+  t.batch = B;
+  t.n = int1 ? K / 32 : K;
+  t.m_chunk = kTileRows;
+  t.n_chunk = int1 ? (size_t)k_per_tile(kInt1) / 32 : (size_t)k_per_tile(input_type);
+  t.elem_bytes = int1 ? 4 : bits_of(input_type) / 8;
+  t.interleaved = (axis == kInterleaved);
+  t.in = src_a;
+  t.out = ws_a;
+  t.m = M;
+  hipError_t e = launch_transpose(t, s);
+  t.in = src_b;
+  t.out = ws_b;
+  t.m = N;
+  if (e == hipSuccess) e = launch_transpose(t, s);
+  if (e != hipSuccess) return fail_hip(e, "transpose kernel launch");
+  GemmParams p;
+  fill_gemm_params(&g, ws_a, ws_b, d_c, &p);
+  e = int1 ? launch_gemm_int1(p, s) : launch_gemm_mfma(p, s);
+  if (e != hipSuccess) return fail_hip(e, "GEMM kernel launch");
+  return CCGLIB_OK;
+}
+
+}  // extern "C"

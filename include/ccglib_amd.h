@@ -207,6 +207,37 @@ CCGLIB_API int ccglib_pipeline_run_host(ccglib_pipeline_t pipeline,
                                         void *h_c);
 CCGLIB_API int ccglib_pipeline_destroy(ccglib_pipeline_t pipeline);
 
+/* ------------------------------------------------------------------------
+ * The pipeline as one stateless call that allocates nothing.
+ * No counterpart in the reference. It is for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc. ccglib_pipeline_create allocates the scratch of its
+ * object (the packed and transposed copies of A and B); this call does the
+ * work of create + run + destroy with that scratch in a static device array
+ * of CCGLIB_AMD_STATIC_SCRATCH_BYTES, which every GPU the library's code is
+ * loaded on holds until the process ends. It calls no hipMalloc / hipFree (nor
+ * their stream-ordered forms) and creates no host objects.
+ *   - Arguments as ccglib_pipeline_create followed by those of
+ *     ccglib_pipeline_run; only enqueues on `stream`.
+ *   - Route: [1-bit interleaved input: pack each batch] -> transpose A and B
+ *     into the tiled layout (1-bit planar input: bytes packed straight into
+ *     1-bit tiles) -> GEMM on the tiles, whatever the variant. The process-wide
+ *     options do not apply.
+ *   - The tiled copies (rows padded to 128, K to the chunk of get_dimensions)
+ *     plus the packed copies must fit the array; otherwise
+ *     CCGLIB_ERROR_UNSUPPORTED and nothing is enqueued. K must be positive
+ *     (1-bit input: a multiple of 32).
+ *   - All calls on one GPU share the array: calls whose kernels may overlap
+ *     (different streams, no dependency) race. Calls on one stream are safe.
+ * ---------------------------------------------------------------------- */
+#define CCGLIB_AMD_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+CCGLIB_API int ccglib_pipeline_run_static(
+    size_t B, size_t M, size_t N, size_t K, int device, void *stream,
+    int input_complex_axis_location, int output_complex_axis_location,
+    int a_mem_order, int b_mem_order, int c_mem_order, int input_type,
+    int output_type, int variant, float alpha_re, float alpha_im, float beta_re,
+    float beta_im, const void *d_a, const void *d_b, void *d_c);
+
 #ifdef __cplusplus
 }
 #endif
