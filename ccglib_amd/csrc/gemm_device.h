@@ -118,27 +118,71 @@ __device__ __forceinline__ unsigned xcd_remap(unsigned wg, unsigned total) {
 }
 
 
+// n / d for wave-uniform n < 2^20 through the float reciprocal: the product is within 0.2 of
+// the true quotient there (23-bit reciprocal, 24-bit product), so truncation is
+// off by at most one, which the remainder shows. An integer division by a
+// run-time value costs several times as many instructions on this target.
+__device__ __forceinline__ unsigned small_div(unsigned n, unsigned d, unsigned *rem) {
+  // (n and d are the same in every lane; the float arithmetic runs on the vector
+  // ALU, and the result goes back to a scalar register)
+  unsigned q = (unsigned)__builtin_amdgcn_readfirstlane(
+      (int)(unsigned)((float)n * __builtin_amdgcn_rcpf((float)d)));
+  unsigned r = n - q * d;
+  if ((int)r < 0) {
+    --q;
+    r += d;
+  } else if (r >= d) {
+    ++q;
+    r -= d;
+  }
+  *rem = r;
+  return q;
+}
+
 // Splits the logical tile id into (batch, block_x, block_y). Inside a batch,
 // tiles are walked in groups of 4 block rows with y fastest, so the 32
 // consecutive tiles that one XCD works on touch 4 Y panels and 8 X panels.
+// (Persistent blocks call this once per C tile, between two K iterations: with
+// fewer than 2^20 tiles in all it takes the short divisions above.)
 struct TileCoord {
   unsigned b, block_x, block_y;
 };
 __device__ __forceinline__ TileCoord tile_coord(const KernelArgs &args, unsigned wg) {
   const unsigned per_batch = args.blocks_x * args.blocks_y;
-  const unsigned logical = xcd_remap(wg, per_batch * args.batch);
+  const unsigned total = per_batch * args.batch;
+  const unsigned logical = xcd_remap(wg, total);
+  const bool small = total < (1u << 20);
   TileCoord tc;
-  tc.b = logical / per_batch;
-  unsigned t = logical % per_batch;
+  unsigned t;
+  if (small) {
+    tc.b = small_div(logical, per_batch, &t);
+  } else {
+    tc.b = logical / per_batch;
+    t = logical % per_batch;
+  }
   constexpr unsigned GROUP = 4;
   const unsigned group_size = GROUP * args.blocks_x;
-  const unsigned g = t / group_size;
+  unsigned in_group;
+  const unsigned g = small ? small_div(t, group_size, &in_group) : t / group_size;
+  if (!small) in_group = t - g * group_size;
   const unsigned first_y = g * GROUP;
   const unsigned rows_in_group =
       (args.blocks_y - first_y) < GROUP ? (args.blocks_y - first_y) : GROUP;
-  t -= g * group_size;
-  tc.block_y = first_y + t % rows_in_group;
-  tc.block_x = t / rows_in_group;
+  if (rows_in_group == GROUP) {
+    tc.block_y = first_y + in_group % GROUP;
+    tc.block_x = in_group / GROUP;
+  } else if (small) {
+    unsigned y;
+    tc.block_x = small_div(in_group, rows_in_group, &y);
+    tc.block_y = first_y + y;
+  } else {
+    tc.block_y = first_y + in_group % rows_in_group;
+    tc.block_x = in_group / rows_in_group;
+  }
+  // wave-uniform by construction; say so, so that addresses built from them stay scalar
+  tc.b = (unsigned)__builtin_amdgcn_readfirstlane((int)tc.b);
+  tc.block_x = (unsigned)__builtin_amdgcn_readfirstlane((int)tc.block_x);
+  tc.block_y = (unsigned)__builtin_amdgcn_readfirstlane((int)tc.block_y);
   return tc;
 }
 

@@ -240,7 +240,8 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
 // xo[i] is the lane's offset of the X fragment of tile i. XT: the operand roles
 // of the MFMA are exchanged (Y supplies the instruction's "A" rows, X its "B"
 // columns), which transposes what a lane holds of every 16 x 16 tile.
-template <int DT, int BX, int BY, bool XT, typename Mid>
+// FIRST: the first K tile of a C tile; the sums start from zero.
+template <int DT, int BX, int BY, bool XT, bool FIRST, typename Mid>
 __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&xo)[4], int y_frag_off,
                                                  float4_t (&acc_re)[4][4], float4_t (&acc_im)[4][4],
                                                  Mid &&mid) {
@@ -253,6 +254,7 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&x
   auto mm = [](const Fragment<DT> &x, const Fragment<DT> &y, float4_t acc) {
     return XT ? mfma<DT>(y, x, acc) : mfma<DT>(x, y, acc);
   };
+  auto c0 = [](const float4_t &acc) { return FIRST ? float4_t{0.f, 0.f, 0.f, 0.f} : acc; };
   constexpr int ROW16 = 16 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
 #define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
   Fragment<DT> xr[4], xi[4], yr, yi, yin, yr_next, yi_next;
@@ -261,28 +263,28 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&x
   xr[1] = rd(xo[1]);
   xr[2] = rd(xo[2]);
   CCGLIB_PIN;
-  acc_re[0][0] = mm(xr[0], yr, acc_re[0][0]);
+  acc_re[0][0] = mm(xr[0], yr, c0(acc_re[0][0]));
   xr[3] = rd(xo[3]);
   CCGLIB_PIN;
-  acc_re[0][1] = mm(xr[1], yr, acc_re[0][1]);
+  acc_re[0][1] = mm(xr[1], yr, c0(acc_re[0][1]));
   yi = rd(y_frag_off + YP);
   CCGLIB_PIN;
-  acc_re[0][2] = mm(xr[2], yr, acc_re[0][2]);
+  acc_re[0][2] = mm(xr[2], yr, c0(acc_re[0][2]));
   xi[0] = rd(xo[0] + XP);
   CCGLIB_PIN;
-  acc_re[0][3] = mm(xr[3], yr, acc_re[0][3]);
+  acc_re[0][3] = mm(xr[3], yr, c0(acc_re[0][3]));
   xi[1] = rd(xo[1] + XP);
   CCGLIB_PIN;
-  acc_im[0][0] = mm(xr[0], yi, acc_im[0][0]);
+  acc_im[0][0] = mm(xr[0], yi, c0(acc_im[0][0]));
   xi[2] = rd(xo[2] + XP);
   CCGLIB_PIN;
-  acc_im[0][1] = mm(xr[1], yi, acc_im[0][1]);
+  acc_im[0][1] = mm(xr[1], yi, c0(acc_im[0][1]));
   xi[3] = rd(xo[3] + XP);
   CCGLIB_PIN;
-  acc_im[0][2] = mm(xr[2], yi, acc_im[0][2]);
+  acc_im[0][2] = mm(xr[2], yi, c0(acc_im[0][2]));
   yin = negate<DT>(yi);
   CCGLIB_PIN;
-  acc_im[0][3] = mm(xr[3], yi, acc_im[0][3]);
+  acc_im[0][3] = mm(xr[3], yi, c0(acc_im[0][3]));
   yr_next = rd(y_frag_off + ROW16);
   CCGLIB_PIN;
   acc_re[0][0] = mm(xi[0], yin, acc_re[0][0]);
@@ -306,16 +308,16 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&x
     // from one MFMA to the next only one of the two operands changes (measured 1-2 %
     // faster on random data than four MFMAs per Y fragment in a row: the part is
     // power limited, and this order toggles fewer operand bits)
-    acc_re[j][0] = mm(xr[0], yr, acc_re[j][0]);
-    acc_im[j][0] = mm(xr[0], yi, acc_im[j][0]);
-    acc_im[j][1] = mm(xr[1], yi, acc_im[j][1]);
-    acc_re[j][1] = mm(xr[1], yr, acc_re[j][1]);
+    acc_re[j][0] = mm(xr[0], yr, c0(acc_re[j][0]));
+    acc_im[j][0] = mm(xr[0], yi, c0(acc_im[j][0]));
+    acc_im[j][1] = mm(xr[1], yi, c0(acc_im[j][1]));
+    acc_re[j][1] = mm(xr[1], yr, c0(acc_re[j][1]));
     if (j < 3) yr_next = rd(y_frag_off + (j + 1) * ROW16);
     CCGLIB_PIN;
-    acc_re[j][2] = mm(xr[2], yr, acc_re[j][2]);
-    acc_im[j][2] = mm(xr[2], yi, acc_im[j][2]);
-    acc_im[j][3] = mm(xr[3], yi, acc_im[j][3]);
-    acc_re[j][3] = mm(xr[3], yr, acc_re[j][3]);
+    acc_re[j][2] = mm(xr[2], yr, c0(acc_re[j][2]));
+    acc_im[j][2] = mm(xr[2], yi, c0(acc_im[j][2]));
+    acc_im[j][3] = mm(xr[3], yi, c0(acc_im[j][3]));
+    acc_re[j][3] = mm(xr[3], yr, c0(acc_re[j][3]));
     if (j < 3) yi_next = rd(y_frag_off + YP + (j + 1) * ROW16);
     CCGLIB_PIN;
     acc_im[j][0] = mm(xi[0], yr, acc_im[j][0]);
@@ -1408,12 +1410,14 @@ __device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
 #pragma clang diagnostic pop
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER,
-          int MS, int XTM>
+          int MS, bool XT, int XSLOTS>
 __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void complex_gemm_mfma_dtl(
     const KernelArgs args) {
   constexpr int NWX = BX / WX, NWY = BY / WY, NW = NWX * NWY;
   constexpr int TX = WX / MS, TY = WY / MS;          // MFMA tiles of a wave
-  constexpr int KPM = MS == 32 ? 1 : DtypeTraits<DT>::kTilesPerMfma;
+  static_assert(MS == 32 || DtypeTraits<DT>::kTilesPerMfma == 1,
+                "one K tile per iteration: fp8 input runs on the 32-row MFMA here");
+  constexpr int KPM = 1;
   static_assert(MS == 16 || LOADER != kLoadInterleavedVec || DtypeTraits<DT>::kElemBytes == 1,
                 "interleaved operands on the 32-row MFMAs: 8-bit input only");
   // interleaved operands: one plane of (re, im) rows
@@ -1423,16 +1427,14 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   constexpr int RB = IL ? 128 : kTileRowBytes;      // bytes of a row in one slot
   constexpr int RPB = 1024 / RB;                    // rows moved by one 1 KiB copy instruction
   constexpr int CPR = RB / 16;                      // 16-byte chunks per row
-  constexpr int KPI = IL ? 1 : KPM;                 // slots per iteration
-  constexpr int X_BYTES = PLANES * BX * RB;
-  constexpr int SLOT_BYTES = X_BYTES + PLANES * BY * RB;
-  constexpr int ROW_BLOCKS = SLOT_BYTES / 1024;     // 1 KiB each: 16 rows x 64 bytes or 8 x 128
-  constexpr int X_ROW_BLOCKS = X_BYTES / 1024;
-  static_assert(ROW_BLOCKS % NW == 0, "row blocks must divide evenly over the waves");
-  constexpr int LPW = ROW_BLOCKS / NW;              // loads per wave per K tile
-  // XTM 0: off; 1: exchanged MFMA roles (below); 2: also the early refill at the
-  // end of a C tile (see the pipeline)
-  constexpr bool XT = XTM != 0, EARLY = XTM == 2;
+  constexpr int X_BYTES = PLANES * BX * RB, Y_BYTES = PLANES * BY * RB;
+  constexpr int SLOT_BYTES = X_BYTES + Y_BYTES;
+  // 1 KiB row blocks (16 rows x 64 bytes or 8 x 128) of the X and the Y part of a K tile
+  constexpr int X_ROW_BLOCKS = X_BYTES / 1024, Y_ROW_BLOCKS = Y_BYTES / 1024;
+  static_assert(X_ROW_BLOCKS % NW == 0 && Y_ROW_BLOCKS % NW == 0,
+                "row blocks must divide evenly over the waves");
+  constexpr int XL = X_ROW_BLOCKS / NW, YL = Y_ROW_BLOCKS / NW;   // loads per wave per K tile
+  constexpr int LPW = XL + YL;
   // XT: the X fragments feed the "B" side of the 16-row MFMA and tile i of a wave
   // holds the columns x = 4 (lane % 16) + i of its 64, so that a lane ends up with
   // 16 consecutive bytes of four C rows per register index and the C stores need no
@@ -1440,13 +1442,28 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   // LDS in the order [4 a + (i ^ a)] <- row 4 a + i, with their 16-byte chunks XORed
   // with 3 (block & 1): fragment reads of rows 4 r + i are then free of bank
   // conflicts (measured), and a copy instruction still moves the contiguous 1 KiB.
-  static_assert(!XT || (MS == 16 && KPM == 1 && TX == 4 && TY == 4 && !IL && WX == 64 &&
-                        X_ROW_BLOCKS % NW == 0 && NW % 2 == 0),
+  static_assert(!XT || (MS == 16 && TX == 4 && TY == 4 && !IL && WX == 64 && NW % 2 == 0 &&
+                        (BX / 16) % 2 == 0),
                 "exchanged roles: 16-row MFMA, 4 x 4 tiles per wave");
-  constexpr int X_LOADS = X_ROW_BLOCKS / NW;        // (XT) the first loads of a wave are X row blocks
-  static_assert(SLOTS % KPI == 0 && SLOTS / KPI >= 2, "ring must hold at least two iterations");
-  constexpr int LEAD = SLOTS / KPI - 1;             // iterations of prefetch distance
-  static_assert((LEAD - 1) * KPI * LPW < 64, "vmcnt range");
+  // The ring. SLOTS K tiles of Y and XSLOTS >= SLOTS K tiles of X: X tiles are
+  // requested XLEAD iterations before their use, Y tiles YLEAD iterations. With
+  // equal counts a slot is [X | Y] as one piece of LDS; with more X slots the
+  // two rings lie one after the other (X is then the operand to make the narrower
+  // one: more of its K tiles fit, and a longer wait for memory is covered).
+  static_assert(SLOTS >= 2 && XSLOTS >= SLOTS, "ring must hold at least two iterations");
+  constexpr bool SPLIT = XSLOTS != SLOTS;
+  constexpr int XLEAD = XSLOTS - 1, YLEAD = SLOTS - 1;
+  // The counter of outstanding copies retires in order. In every iteration a wave
+  // requests its Y blocks first and then its X blocks; the K tile of iteration k is
+  // complete when nothing older than the last request for it is outstanding, which
+  // leaves the requests of the YLEAD - 1 iterations since, and the X blocks that
+  // followed Y(k) in its own iteration when X runs further ahead.
+  constexpr int kOutstandingOk = (XLEAD > YLEAD ? XL : 0) + (YLEAD - 1) * LPW;
+  static_assert(kOutstandingOk < 64, "vmcnt range");
+  auto x_slot_off = [](unsigned s) { return SPLIT ? s * X_BYTES : s * SLOT_BYTES; };
+  auto y_slot_off = [](unsigned s) {
+    return SPLIT ? XSLOTS * X_BYTES + s * Y_BYTES : s * SLOT_BYTES + X_BYTES;
+  };
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -1455,23 +1472,19 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int wx = wave % NWX, wy = wave / NWX;
   // slots along K (the host counts 64-byte pieces of a row)
   const unsigned k_tiles = IL ? (args.k_tiles + 1) / 2 : args.k_tiles;
-  const unsigned k_tiles_padded = (k_tiles + KPI - 1) / KPI * KPI;
   const unsigned total = args.blocks_x * args.blocks_y * args.batch;
   // bytes of one operand row in memory (planar: one plane's row)
   const unsigned row_bytes = IL ? 2 * args.k_bytes : args.k_bytes;
   // ... and the distance between rows (larger when the launch covers a piece of K)
   const unsigned row_stride = IL ? 2 * args.row_stride_bytes : args.row_stride_bytes;
 
-  // ---- this wave's share of the copy: LPW row blocks of every K tile ------
-  // Row block q of a slot: X re, X im, Y re, Y im, 16 rows each. What depends
-  // on the lane (its row and swizzled chunk inside the row block) is the same
-  // for every C tile; the wave-uniform tile pointers are set per C tile.
-  unsigned tile_off[LPW];      // wave-uniform: the row block inside its operand tile
+  // ---- this wave's share of the copy: XL + YL row blocks of every K tile --
+  // Row block q of an operand's part of a K tile: re plane, im plane, 16 rows
+  // each. What depends on the lane (its row and swizzled chunk inside the row
+  // block) is the same for every C tile; the wave-uniform tile pointers are set
+  // per C tile.
   const unsigned lane_off = (lane >> 2) * kTileRowBytes +
                             (((lane & 3) ^ (MS == 32 ? (lane >> 4) & 3 : (lane >> 3) & 3)) * 16);
-  unsigned lds_dst[LPW];       // wave-uniform: LDS byte address inside slot 0
-  const char *src[LPW];        // wave-uniform: K tile 0 of the operand tile
-  const char *lane_src[LPW];   // planar layout: this lane's chunk of K tile 0
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
   const int r = lane / CPR;                                   // row inside the row block
   // chunk that belongs at lane*16: the XOR pattern that makes the fragment
@@ -1487,89 +1500,116 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
   const int xt_row = 4 * (lane >> 4) + (((lane >> 2) & 3) ^ (lane >> 4));
   const int xt_chunk = (lane & 3) ^ (3 * (wave & 1));
   const unsigned lane_off_x = XT ? xt_row * kTileRowBytes + xt_chunk * 16 : lane_off;
-  {
+
+  // One operand's side of the copy: where its next K tile comes from. The copy
+  // walks the same sequence of C tiles as the math, X ahead of Y when its ring
+  // is deeper; past the last C tile it re-reads the last one (never used).
+  struct Stream {
+    unsigned tile, kt;          // C tile and K tile of the request issued last
+  };
+  Stream xs{blockIdx.x, 0}, ys{blockIdx.x, 0};
+  unsigned x_tile_off[XL], y_tile_off[YL];   // wave-uniform: the row block inside its operand tile
+  unsigned x_lds[XL], y_lds[YL];             // wave-uniform: LDS byte address inside slot 0 of the ring
+  const char *x_src[XL], *y_src[YL];         // wave-uniform: K tile 0 of the operand tile (tiled layout)
+  const char *x_lane_src[XL], *y_lane_src[YL];   // planar layouts: this lane's chunk of K tile 0
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int q = i * NW + wave;
-      const bool is_x = q < X_ROW_BLOCKS;
-      const int qq = is_x ? q : q - X_ROW_BLOCKS;
-      const int rows = is_x ? BX : BY;
-      const int plane = qq / (rows / RPB), rb = qq % (rows / RPB);
-      // inside the operand tile: the lane's part is the same for every row block
-      tile_off[i] = plane * kTilePlaneBytes + ((rb * RPB) % kTileRows) * kTileRowBytes;
-      lds_dst[i] = lds_base + q * 1024;
-    }
+  for (int i = 0; i < XL; ++i) {
+    const int q = i * NW + wave, plane = q / (BX / RPB), rb = q % (BX / RPB);
+    x_tile_off[i] = plane * kTilePlaneBytes + ((rb * RPB) % kTileRows) * kTileRowBytes;
+    x_lds[i] = lds_base + x_slot_off(0) + q * 1024;
   }
-  // The copy runs LEAD iterations ahead of the math and walks the same
-  // sequence of C tiles; past the last one it reads the zero tile.
-  unsigned load_tile = blockIdx.x, load_kt = 0;
-  auto point_at = [&](unsigned vt) {
-    if (vt < total) {
-      const TileCoord tc = tile_coord(args, vt);
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) {
-        const int q = i * NW + wave;
-        const bool is_x = q < X_ROW_BLOCKS;
-        const int qq = is_x ? q : q - X_ROW_BLOCKS;
-        const int rows = is_x ? BX : BY;
-        const int plane = qq / (rows / RPB), rb = qq % (rows / RPB);
-        const unsigned row0 = (is_x ? tc.block_x * BX : tc.block_y * BY) + rb * RPB;
-        const char *op = is_x ? args.x + (size_t)tc.b * args.x_batch_bytes
-                              : args.y + (size_t)tc.b * args.y_batch_bytes;
-        if constexpr (LOADER == kLoadTiled) {
-          const unsigned tiles = is_x ? args.x_tiles : args.y_tiles;
-          unsigned tile = row0 / kTileRows;
-          tile = tile < tiles ? tile : tiles - 1;   // rows past the end: never stored
-          src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes;
-        } else {
-          const unsigned total_rows = is_x ? args.nx : args.ny;
-          const bool xt = XT && is_x;
-          unsigned row = row0 + (xt ? xt_row : r);
-          row = row < total_rows ? row : total_rows - 1;   // likewise
-          lane_src[i] = op + ((size_t)plane * total_rows + row) * row_stride +
-                        (xt ? xt_chunk : c_of(rb)) * 16;
-        }
+  for (int i = 0; i < YL; ++i) {
+    const int q = i * NW + wave, plane = q / (BY / RPB), rb = q % (BY / RPB);
+    y_tile_off[i] = plane * kTilePlaneBytes + ((rb * RPB) % kTileRows) * kTileRowBytes;
+    y_lds[i] = lds_base + y_slot_off(0) + q * 1024;
+  }
+  // Points one side of the copy at the operand tile of C tile vt.
+  auto point_x = [&](unsigned vt) {
+    if (vt >= total) return;
+    const TileCoord tc = tile_coord(args, vt);
+    const char *op = args.x + (size_t)tc.b * args.x_batch_bytes;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int q = i * NW + wave, plane = q / (BX / RPB), rb = q % (BX / RPB);
+      const unsigned row0 = tc.block_x * BX + rb * RPB;
+      if constexpr (LOADER == kLoadTiled) {
+        unsigned tile = row0 / kTileRows;
+        tile = tile < args.x_tiles ? tile : args.x_tiles - 1;   // rows past the end: never stored
+        x_src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes;
+      } else {
+        unsigned row = row0 + (XT ? xt_row : r);
+        row = row < args.nx ? row : args.nx - 1;   // likewise
+        x_lane_src[i] = op + ((size_t)plane * args.nx + row) * row_stride +
+                        (XT ? xt_chunk : c_of(rb)) * 16;
       }
     }
   };
-  // issue_copies: straight-line code (it is placed between MFMAs, and a
-  // branch there would let the compiler sink those MFMAs below it);
-  // advance_copy: the bookkeeping, with the branches of the tile change.
-  auto issue_copies = [&](int slot) {
-    // Past the last C tile the copy re-reads the last one (never used); only K
-    // tiles past the end of K, whose contents enter the sums, read zeros.
-    if constexpr (LOADER == kLoadTiled) {
-      const bool real = (KPI == 1) || (load_kt < k_tiles);
+  auto point_y = [&](unsigned vt) {
+    if (vt >= total) return;
+    const TileCoord tc = tile_coord(args, vt);
+    const char *op = args.y + (size_t)tc.b * args.y_batch_bytes;
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) {
-        const char *base = real ? src[i] + (size_t)load_kt * kTileBytes + tile_off[i] : g_zero_tile;
-        load_1k_to_lds(base, (XT && i < X_LOADS) ? lane_off_x : lane_off,
-                       lds_dst[i] + slot * SLOT_BYTES);
-      }
-    } else {
-      // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
-#pragma unroll
-      for (int i = 0; i < LPW; ++i) {
-        const int q = i * NW + wave;
-        const int rb = (q < X_ROW_BLOCKS ? q : q - X_ROW_BLOCKS) % ((q < X_ROW_BLOCKS ? BX : BY) / RPB);
-        const int chunk = (XT && q < X_ROW_BLOCKS) ? xt_chunk : c_of(rb);
-        const bool inside = (load_kt * RB + chunk * 16 + 16 <= row_bytes);
-        const char *p = inside ? lane_src[i] + (size_t)load_kt * RB
-                               : g_zero_tile + lane * 16;
-        load_1k_to_lds_by_lane(p, lds_dst[i] + slot * SLOT_BYTES);
+    for (int i = 0; i < YL; ++i) {
+      const int q = i * NW + wave, plane = q / (BY / RPB), rb = q % (BY / RPB);
+      const unsigned row0 = tc.block_y * BY + rb * RPB;
+      if constexpr (LOADER == kLoadTiled) {
+        unsigned tile = row0 / kTileRows;
+        tile = tile < args.y_tiles ? tile : args.y_tiles - 1;
+        y_src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes;
+      } else {
+        unsigned row = row0 + r;
+        row = row < args.ny ? row : args.ny - 1;
+        y_lane_src[i] = op + ((size_t)plane * args.ny + row) * row_stride + c_of(rb) * 16;
       }
     }
   };
-  auto advance_copy = [&] {
-    if (++load_kt == k_tiles_padded) {
-      load_kt = 0;
-      load_tile += gridDim.x;
-      point_at(load_tile);
+  // issue_*: straight-line code (it is placed between MFMAs, and a branch there
+  // would let the compiler sink those MFMAs below it); advance_*: the
+  // bookkeeping, with the branches of the tile change.
+  auto issue_x = [&](unsigned slot) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const unsigned dst = x_lds[i] + (x_slot_off(slot) - x_slot_off(0));
+      if constexpr (LOADER == kLoadTiled) {
+        load_1k_to_lds(x_src[i] + (size_t)xs.kt * kTileBytes + x_tile_off[i], lane_off_x, dst);
+      } else {
+        // rows are whole 16-byte chunks: a chunk is either inside K or reads zeros
+        const int q = i * NW + wave, rb = q % (BX / RPB);
+        const int chunk = XT ? xt_chunk : c_of(rb);
+        const bool inside = (xs.kt * RB + chunk * 16 + 16 <= row_bytes);
+        load_1k_to_lds_by_lane(inside ? x_lane_src[i] + (size_t)xs.kt * RB : g_zero_tile + lane * 16,
+                               dst);
+      }
     }
   };
-  auto issue_next = [&](int slot) {
-    issue_copies(slot);
-    advance_copy();
+  auto issue_y = [&](unsigned slot) {
+#pragma unroll
+    for (int i = 0; i < YL; ++i) {
+      const unsigned dst = y_lds[i] + (y_slot_off(slot) - y_slot_off(0));
+      if constexpr (LOADER == kLoadTiled) {
+        load_1k_to_lds(y_src[i] + (size_t)ys.kt * kTileBytes + y_tile_off[i], lane_off, dst);
+      } else {
+        const int q = i * NW + wave, rb = q % (BY / RPB);
+        const bool inside = (ys.kt * RB + c_of(rb) * 16 + 16 <= row_bytes);
+        load_1k_to_lds_by_lane(inside ? y_lane_src[i] + (size_t)ys.kt * RB : g_zero_tile + lane * 16,
+                               dst);
+      }
+    }
+  };
+  auto advance_x = [&] {
+    if (++xs.kt == k_tiles) {
+      xs.kt = 0;
+      xs.tile += gridDim.x;
+      point_x(xs.tile);
+    }
+  };
+  auto advance_y = [&] {
+    if (++ys.kt == k_tiles) {
+      ys.kt = 0;
+      ys.tile += gridDim.x;
+      point_y(ys.tile);
+    }
   };
 
   const int frag_lane_off = swizzled_row_offset(lane & 15, lane >> 4);
@@ -1618,87 +1658,77 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
                          args.c_vector_ok && (args.nx % 4 == 0);
 
   // ---- pipeline ----------------------------------------------------------
-  point_at(load_tile);
-  // With one slot per iteration the bookkeeping of the copy (advance_copy, which
-  // branches) is done at the top of an iteration for the copies issued inside it,
-  // so that nothing but straight-line code follows the barrier.
+  point_x(xs.tile);
+  point_y(ys.tile);
+  // The bookkeeping of the copy (advance_*, which branches) is done at the top of
+  // an iteration for the copies issued inside it, so that nothing but
+  // straight-line code follows the barrier. Before the first iteration: the
+  // requests that iterations -XLEAD .. -1 would have made, in their order.
 #pragma unroll
-  for (int t = 0; t < LEAD * KPI; ++t) {
-    if constexpr (KPI == 1) {
-      if (t > 0) advance_copy();
-      issue_copies(t);
-    } else {
-      issue_next(t);
+  for (int t = -XLEAD; t < 0; ++t) {
+    if (t + YLEAD >= 0) {
+      if (t + YLEAD > 0) advance_y();
+      issue_y(t + YLEAD);
     }
+    if (t + XLEAD > 0) advance_x();
+    issue_x(t + XLEAD);
   }
-  unsigned slot = 0;                       // first slot of the current iteration
-  const unsigned iters = k_tiles_padded / KPI;
-  // (EARLY) store instructions of the fast epilogue of one wave, and whether the
-  // previous tile's epilogue was that one
-  constexpr int kFastStores = 2 * TY * 4;
-  static_assert(!EARLY || (LEAD == 2 && KPI == 1 && kFastStores + LPW < 64), "early refill");
-  bool stores_in_flight = false;
+  unsigned x_slot = 0, y_slot = 0;         // slots of the current iteration
+  const unsigned iters = k_tiles;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
     typename AccType<MS>::type acc_re[TY][TX], acc_im[TY][TX];
+    // (the hand-ordered step of the 16-row MFMAs starts its first iteration from zero itself)
+    constexpr bool kStepClears = !IL && DT != kInt1 && MS == 16 && TX == 4 && TY == 4;
+    static_assert(!SPLIT || kStepClears, "separate X and Y rings: hand-ordered 16-row step only");
+    if constexpr (!kStepClears) {
 #pragma unroll
-    for (int j = 0; j < TY; ++j) {
+      for (int j = 0; j < TY; ++j) {
 #pragma unroll
-      for (int i = 0; i < TX; ++i) {
-        acc_re[j][i] = 0.f;
-        acc_im[j][i] = 0.f;
+        for (int i = 0; i < TX; ++i) {
+          acc_re[j][i] = 0.f;
+          acc_im[j][i] = 0.f;
+        }
       }
     }
     for (unsigned it = 0; it < iters; ++it) {
-      // (EARLY) the first iteration of a C tile after the block's first issues no
-      // copies: the K tile it would fetch was requested before the previous
-      // tile's C stores
-      const bool no_refill = EARLY && it == 0 && vt != blockIdx.x;
-      if constexpr (KPI == 1) {
-        if (!no_refill) advance_copy();
-      }
-      // After the first C tile, the K tiles of the first LEAD iterations were
+      advance_y();
+      advance_x();
+      // After the first C tile, the K tiles of the first YLEAD iterations were
       // already waited for before the previous epilogue (see below), so these
       // iterations only need the barrier; waiting on the counter here would
       // wait for the previous tile's C stores, which are younger than them.
-      if (vt != blockIdx.x && it < (unsigned)LEAD) {
+      if (vt != blockIdx.x && it < (unsigned)YLEAD) {
         asm volatile("s_barrier" ::: "memory");
-      } else if (EARLY && vt != blockIdx.x && it == (unsigned)LEAD && stores_in_flight) {
-        // the K tile of this iteration was requested before the C stores of the
-        // previous tile: they and this wave's copies of the next K tile may still be
-        // in flight (the counter retires in order)
-        wait_vmcnt_then_barrier<kFastStores + (LEAD - 1) * KPI * LPW>();
       } else {
-        wait_vmcnt_then_barrier<(LEAD - 1) * KPI * LPW>();
+        wait_vmcnt_then_barrier<kOutstandingOk>();
       }
       // the slots of the previous iteration are free now: refill them with the
-      // K tiles that are LEAD iterations ahead (of this C tile or the next)
-      unsigned refill = slot + LEAD * KPI;
-      refill = refill >= SLOTS ? refill - SLOTS : refill;
+      // K tiles that are XLEAD / YLEAD iterations ahead (of this C tile or the next)
+      unsigned x_refill = x_slot + XLEAD, y_refill = y_slot + YLEAD;
+      x_refill = x_refill >= XSLOTS ? x_refill - XSLOTS : x_refill;
+      y_refill = y_refill >= SLOTS ? y_refill - SLOTS : y_refill;
       // The copy instructions go out after the first group of MFMAs: right
       // after the barrier every wave of the block would otherwise be busy with
       // their address arithmetic and the matrix cores would have nothing to do.
       auto refill_slots = [&] {
-        if constexpr (KPI == 1) {
-          issue_copies(refill);
-        } else {
-#pragma unroll
-          for (int u = 0; u < KPI; ++u) issue_next(refill + u);
-        }
+        issue_y(y_refill);
+        issue_x(x_refill);
       };
+      const char *slot_ptr = lds + x_slot_off(x_slot);
+      // (the fragment offsets of Y count from the start of an [X | Y] slot)
+      const int y_shift = (int)y_slot_off(y_slot) - (int)x_slot_off(x_slot) - X_BYTES;
       if constexpr (IL && MS == 32) {
         static_assert(TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
-        mma_step32_interleaved<DT, BX, BY>(lds + slot * SLOT_BYTES, xil32_off, yil32_off, acc_re,
-                                           acc_im, refill_slots);
+        mma_step32_interleaved<DT, BX, BY>(slot_ptr, xil32_off, yil32_off, acc_re, acc_im,
+                                           refill_slots);
       } else if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
-        mma_step_interleaved_ordered<DT, BX, BY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
-                                                 acc_im, refill_slots);
+        mma_step_interleaved_ordered<DT, BX, BY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
+                                                 refill_slots);
       } else if constexpr (IL) {
-        mma_step_interleaved<DT, BX, BY, TX, TY>(lds + slot * SLOT_BYTES, xil_off, yil_off, acc_re,
-                                                 acc_im, refill_slots);
+        mma_step_interleaved<DT, BX, BY, TX, TY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
+                                                 refill_slots);
       } else {
-        const char *tile[KPM];
-#pragma unroll
-        for (int u = 0; u < KPM; ++u) tile[u] = lds + (slot + u) * SLOT_BYTES;
+        const char *tile[KPM] = {slot_ptr};
         if constexpr (DT == kInt1) {
           static_assert(MS == 32 && TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
           mma_step32_bits<BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
@@ -1706,58 +1736,49 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
           mma_step32_ordered<DT, BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
         } else if constexpr (MS == 32) {
           mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
-        } else if constexpr (KPM == 1 && TX == 4 && TY == 4) {
-          if (no_refill) {
-            mma_step_ordered<DT, BX, BY, XT>(tile[0], xo, y_frag_off, acc_re, acc_im, [] {});
+        } else if constexpr (TX == 4 && TY == 4) {
+          // (the first iteration of a C tile starts its sums from zero instead of
+          // from accumulators that would have to be cleared first)
+          if (it == 0) {
+            mma_step_ordered<DT, BX, BY, XT, true>(tile[0], xo, y_frag_off + y_shift, acc_re, acc_im,
+                                                   refill_slots);
           } else {
-            mma_step_ordered<DT, BX, BY, XT>(tile[0], xo, y_frag_off, acc_re, acc_im, refill_slots);
+            mma_step_ordered<DT, BX, BY, XT, false>(tile[0], xo, y_frag_off + y_shift, acc_re, acc_im,
+                                                    refill_slots);
           }
         } else {
           mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
         }
       }
-      slot += KPI;
-      slot = slot >= SLOTS ? slot - SLOTS : slot;
+      x_slot = x_slot + 1 == XSLOTS ? 0 : x_slot + 1;
+      y_slot = y_slot + 1 == SLOTS ? 0 : y_slot + 1;
     }
     // The stores below are not waited for here: they drain while the next C
     // tile is being computed. The counter cannot tell loads from stores, so
     // the next tile's first K tiles, which are already on their way, are waited
-    // for now; the first wait that has to include the stores then comes LEAD
+    // for now; the first wait that has to include the stores then comes YLEAD
     // iterations into the next tile.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const TileCoord tc = tile_coord(args, vt);
     const unsigned x_wave = tc.block_x * BX + wx * WX, y_wave = tc.block_y * BY + wy * WY;
     bool staged = false;
-    if constexpr (EARLY) {
-      // The slot consumed last is free once every wave has left the K loop. The K
-      // tile that the next iteration would request is requested now, ahead of
-      // the C stores: the memory pipeline of the compute unit works in order, and
-      // a request behind 256 KiB of stores comes back after the iteration that
-      // needs it.
-      unsigned free_slot = slot + LEAD * KPI;
-      free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
-      asm volatile("s_barrier" ::: "memory");
-      advance_copy();
-      issue_copies(free_slot);
-    }
     if constexpr (XT) {
       // the accumulators already hold whole row segments
       if (staged_ok && !args.c_interleaved && x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
         store_wave_tile_rows<TOUT, TY>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
-        stores_in_flight = true;
       } else {
         store_wave_tile<TOUT, TX, TY, kAcc16T>(args, tc.b, x_wave, y_wave, lane, acc_re, acc_im);
-        stores_in_flight = false;
       }
       staged = true;
     }
     if constexpr (!XT && MS == 16 && TOUT == kFloat32 && TX == 4 &&
-                  NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
+                  !SPLIT && NW * kStagePatchBytes <= SLOT_BYTES) {
       if (staged_ok) {
         // The slot consumed last is free until the next refill, but other waves
         // may still be reading it: one barrier, then every wave uses its own
         // patch of it. (Uniform per block, so the barrier is safe.)
-        unsigned free_slot = slot + LEAD * KPI;
+        // ([X | Y] slots here: the rings are one)
+        unsigned free_slot = y_slot + YLEAD;
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
@@ -1772,9 +1793,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     if constexpr (!XT && MS == 16 && (TOUT == kFloat16 || TOUT == kBfloat16) && TX == 4 &&
-                  NW * kStagePatchBytes <= KPI * SLOT_BYTES) {
+                  !SPLIT && NW * kStagePatchBytes <= SLOT_BYTES) {
       if (staged_ok && !args.c_interleaved && args.nx % 8 == 0) {
-        unsigned free_slot = slot + LEAD * KPI;
+        // ([X | Y] slots here: the rings are one)
+        unsigned free_slot = y_slot + YLEAD;
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
@@ -1786,9 +1808,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       }
     }
     if constexpr (MS == 32 && (TOUT == kFloat32 || TOUT == kInt32) &&
-                  NW * kStagePatch32Bytes <= KPI * SLOT_BYTES) {
+                  !SPLIT && NW * kStagePatch32Bytes <= SLOT_BYTES) {
       if (staged_ok) {
-        unsigned free_slot = slot + LEAD * KPI;
+        // ([X | Y] slots here: the rings are one)
+        unsigned free_slot = y_slot + YLEAD;
         free_slot = free_slot >= SLOTS ? free_slot - SLOTS : free_slot;
         asm volatile("s_barrier" ::: "memory");
         if (x_wave + WX <= args.nx && y_wave + WY <= args.ny) {
@@ -1861,10 +1884,10 @@ inline int compute_units() {
 }
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WPE,
-          int LOADER = kLoadTiled, int MS = 16, int XT = 0>
+          int LOADER = kLoadTiled, int MS = 16, bool XT = false, int XSLOTS = SLOTS>
 hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   constexpr int NTHREADS = 64 * (BX / WX) * (BY / WY);
-  constexpr int LDS_BYTES = SLOTS * 2 * (BX + BY) * kTileRowBytes;
+  constexpr int LDS_BYTES = 2 * (XSLOTS * BX + SLOTS * BY) * kTileRowBytes;
   constexpr int kLdsPerCu = 160 * 1024;
   constexpr int BLOCKS_PER_CU = (kLdsPerCu / LDS_BYTES) < (WPE * 256 / NTHREADS)
                                     ? (kLdsPerCu / LDS_BYTES)
@@ -1874,7 +1897,7 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS, XT>;
+  auto kernel = complex_gemm_mfma_dtl<DT, TOUT, BX, BY, WX, WY, SLOTS, WPE, LOADER, MS, XT, XSLOTS>;
   static std::atomic<bool> lds_allowed[kMaxDevices];
   if (hipError_t e = allow_lds(kernel, LDS_BYTES, lds_allowed)) return e;
   // persistent blocks: as many as are resident at once, each walking C tiles
@@ -1908,8 +1931,8 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     if constexpr (KPM == 1) {
       // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
       return p.variant == kOpt
-                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 2>(p, stream)
-                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, 2>(p, stream);
+                 ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>(p, stream)
+                 : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>(p, stream);
     } else {
       // fp8: the 32x32x64 MFMA takes one K tile per instruction, which lets the
       // same block shape and ring as for 16-bit input fit into LDS

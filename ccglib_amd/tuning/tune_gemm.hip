@@ -38,22 +38,21 @@ struct Config {
 // name: type, block BX x BY, wave WX x WY, ring slots, MFMA rows
 static const std::vector<Config> kConfigs = {
     {"f16 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat16, kFloat32},
-    {"f16 256x128 w64x64 s3 m16 xt1", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 1>, kFloat16, kFloat32},
-    {"f16 256x128 w64x64 s3 m16 xt2", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, 2>, kFloat16, kFloat32},
+    {"f16 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
+    {"f16 128x256 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
+    {"f16 128x256 w64x64 y3 x4 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true, 4>, kFloat16, kFloat32},
     {"f16 256x128 w64x64 s3 m32", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat16, kFloat32},
     {"f16 128x128 w64x64 s2 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"f16 128x128 w64x32 s4 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"bf16 256x128 w64x64 s3 m16", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kBfloat16, kFloat32},
     {"f32 256x128 w64x64 s3 m16", launch_dtl<kFloat32, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat32, kFloat32},
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
-    {"fp8 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat8e4m3, kFloat32},
     {"int1 256x128 w64x64 s3 m32", launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kInt1, kInt32},
     // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
-    {"f16 planar 256x128 w64x64 s3 m16 xt2", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, 2>, kFloat16, kFloat32, kLoadPlanarVec},
+    {"f16 planar 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>, kFloat16, kFloat32, kLoadPlanarVec},
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
-    {"fp8 interleaved 128x128 w64x32 s4 m16", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec, 16>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
     {"fp8 interleaved 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
 };
 
