@@ -4,9 +4,9 @@
 // Stands in for the reference's transpose kernel
 // (kernels/transpose_kernel.cu:50-82), which moves one element pair per
 // thread. This one is bandwidth-shaped: a thread moves 16-byte vectors (both
-// planes of 4 rows), lanes of a wave run along N across tile boundaries, so
-// loads are contiguous runs of 256 bytes per row and stores are contiguous
-// runs of rows inside each output tile. Both sides are streamed once, so the
+// planes of 2 rows), lanes of a wave run along N across tile boundaries, so
+// loads are contiguous runs of 128 or 256 bytes per row and stores are
+// contiguous runs of rows inside each output tile. Both sides are streamed once, so the
 // accesses carry the non-temporal hint (measured +5 to +10 % on this part).
 // A scalar kernel covers shapes whose rows are not whole 16-byte vectors.
 #include "common.h"
@@ -92,21 +92,23 @@ __device__ __forceinline__ void load_ragged(const char *p, size_t plane_stride_b
 }
 
 constexpr int kRowsPerThread = 2;
-constexpr int kVecsPerBlockRow = 16;   // 256 bytes of a row per block
-constexpr int kRowsPerBlock = 16 * kRowsPerThread;
 
-// grid: (ceil(n_vecs_padded / 16), ceil(Mp / 32), B); block: 256 threads as
-// 16 vectors x 16 rows, each thread doing rows r and r+16 (two rows a thread
-// measured best over the operand shapes of the benchmark configurations: one
-// row is as good for 16-bit but slower for 8-bit elements, four are 2-7 %
-// slower, eight halve the rate).
+// grid: (ceil(n_vecs_padded / VPR), ceil(Mp / rows per block), B); block: 256
+// threads as VPR vectors x 256 / VPR rows, each thread doing rows r and
+// r + 256 / VPR (two rows a thread measured best over the operand shapes of the
+// benchmark configurations: one row is as good for 16-bit but slower for 8-bit
+// elements, four are 2-7 % slower, eight halve the rate). VPR is 16 (256 bytes
+// of a row per block) or, for padded rows that are a multiple of 8 but not of
+// 16 vectors, 8: no lanes without work at the end of a row (K = 576 halfs is
+// 72 vectors: with 16 a tenth of the threads would idle).
 // RAGGED: input rows of any length at any element-aligned address (the output
 // tiles still hold whole vectors per row).
-template <int EB, bool INTERLEAVED, bool RAGGED>
+template <int EB, bool INTERLEAVED, bool RAGGED, int VPR>
 __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
   constexpr int V = 16 / EB;  // elements per vector
-  const size_t nvec = (size_t)blockIdx.x * kVecsPerBlockRow + (threadIdx.x & 15);
-  const size_t m_base = (size_t)blockIdx.y * kRowsPerBlock + (threadIdx.x >> 4);
+  constexpr int RS = 256 / VPR;   // rows between the two rows of a thread
+  const size_t nvec = (size_t)blockIdx.x * VPR + (threadIdx.x % VPR);
+  const size_t m_base = (size_t)blockIdx.y * (RS * kRowsPerThread) + (threadIdx.x / VPR);
   const size_t b = blockIdx.z;
   const size_t m_padded = a.m_tiles * a.m_chunk;
   if (nvec >= a.n_vecs_padded) return;
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
   uint4_t re[kRowsPerThread], im[kRowsPerThread];
 #pragma unroll
   for (int i = 0; i < kRowsPerThread; ++i) {
-    const size_t m = m_base + 16 * i;
+    const size_t m = m_base + RS * i;
     re[i] = uint4_t{0, 0, 0, 0};
     im[i] = uint4_t{0, 0, 0, 0};
     if (m < a.m && n_ok) {
@@ -140,7 +142,7 @@ __global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
   }
 #pragma unroll
   for (int i = 0; i < kRowsPerThread; ++i) {
-    const size_t m = m_base + 16 * i;
+    const size_t m = m_base + RS * i;
     if (m < m_padded) {
       const size_t mt = m / a.m_chunk, mr = m % a.m_chunk;
       char *q = a.out + (((b * a.m_tiles + mt) * a.n_tiles + nt) * 2) * plane_bytes +
@@ -196,26 +198,29 @@ hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
   const size_t m_padded = a.m_tiles * a.m_chunk, n_padded = a.n_tiles * a.n_chunk;
   if (p.batch == 0 || m_padded == 0 || n_padded == 0) return hipSuccess;
   // whole vectors per output tile row; the input may be ragged
+  const bool narrow = (n_padded / V) % 16 != 0 && (n_padded / V) % 8 == 0;
+  const size_t vpr = narrow ? 8 : 16, rows_per_block = 256 / vpr * kRowsPerThread;
   const bool out_vec_ok = (p.n_chunk % V == 0) && ((uintptr_t)p.out % 16 == 0) &&
                           ((uintptr_t)p.in % EB == 0) && p.batch <= 65535 &&
-                          ceil_div(m_padded, kRowsPerBlock) <= 65535;
+                          ceil_div(m_padded, rows_per_block) <= 65535;
   const bool in_vec_ok = (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0);
   if (out_vec_ok) {
     a.n_vecs_padded = n_padded / V;
     a.vecs_per_tile_row = p.n_chunk / V;
-    const dim3 grid((unsigned)ceil_div(a.n_vecs_padded, kVecsPerBlockRow),
-                    (unsigned)ceil_div(m_padded, kRowsPerBlock), (unsigned)p.batch);
+    const dim3 grid((unsigned)ceil_div(a.n_vecs_padded, vpr),
+                    (unsigned)ceil_div(m_padded, rows_per_block), (unsigned)p.batch);
+    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, a); };
     if (p.interleaved) {
       if (in_vec_ok) {
-        hipLaunchKernelGGL((transpose_vec<EB, true, false>), grid, dim3(256), 0, stream, a);
+        narrow ? launch(transpose_vec<EB, true, false, 8>) : launch(transpose_vec<EB, true, false, 16>);
       } else {
-        hipLaunchKernelGGL((transpose_vec<EB, true, true>), grid, dim3(256), 0, stream, a);
+        narrow ? launch(transpose_vec<EB, true, true, 8>) : launch(transpose_vec<EB, true, true, 16>);
       }
     } else {
       if (in_vec_ok) {
-        hipLaunchKernelGGL((transpose_vec<EB, false, false>), grid, dim3(256), 0, stream, a);
+        narrow ? launch(transpose_vec<EB, false, false, 8>) : launch(transpose_vec<EB, false, false, 16>);
       } else {
-        hipLaunchKernelGGL((transpose_vec<EB, false, true>), grid, dim3(256), 0, stream, a);
+        narrow ? launch(transpose_vec<EB, false, true, 8>) : launch(transpose_vec<EB, false, true, 16>);
       }
     }
   } else {

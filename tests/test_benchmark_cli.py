@@ -72,3 +72,31 @@ def test_transpose_and_packing_csv():
                 "--csv")
         assert r.returncode == 0, r.stderr
         assert r.stdout.splitlines()[0] == "#N,runtime_ms,gbytes" and len(r.stdout.splitlines()) == 3
+
+
+TUNE = os.path.join(os.path.dirname(HERE), "ccglib_amd", "tuning", "tune_gemm")
+
+
+@pytest.mark.gpu
+def test_tuner_sweeps_its_configurations():
+    """The kernel-configuration sweep (the counterpart of the reference's tuning/tune_gemm.py:316-363)
+    runs every configuration on a small shape and prints one timed line per configuration."""
+    if not os.path.exists(TUNE):
+        pytest.skip("tuner not built")
+    r = subprocess.run([TUNE, "2", "256", "256", "64"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    lines = r.stdout.strip().splitlines()
+    assert lines[0].startswith("configuration") and "B=2 M=256 N=256 K=64" in lines[0]
+    rows = [l for l in lines[1:] if "%" in l]
+    assert len(rows) >= 10
+    # the configurations that the library's dispatch uses are among them
+    names = " | ".join(rows)
+    for want in ("f16 256x128 w64x64 s3 m16 xt", "fp8 256x128 w64x64 s3 m32", "int1 256x128 w64x64 s3 m32",
+                 "f16 planar 256x128 w64x64 s3 m16 xt", "f16 interleaved 256x128 w64x64 s3 m16"):
+        assert want in names, want
+    for l in rows:
+        ms, rate = float(l.split()[-3]), float(l.split()[-2])
+        assert ms > 0 and rate > 0
+    # a filter selects configurations by name
+    r = subprocess.run([TUNE, "2", "256", "256", "64", "bf16"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and all("bf16" in l for l in r.stdout.strip().splitlines()[1:])
