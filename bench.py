@@ -162,10 +162,13 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
     b_t = torch.empty(B * 2 * np_ * kp * bits // 8, dtype=torch.uint8, device="cuda")
     tr_a = cc.Transpose(B, M, K, mb, kc, bits, 0, stream, axis)
     tr_b = cc.Transpose(B, N, K, nb, kc, bits, 0, stream, axis)
-    kernels.append(("transpose_a", lambda s=a_cur: tr_a.Run(s.data_ptr(), a_t.data_ptr()),
-                    2.0 * B * 2 * M * K * bits / 8))
-    kernels.append(("transpose_b", lambda s=b_cur: tr_b.Run(s.data_ptr(), b_t.data_ptr()),
-                    2.0 * B * 2 * N * K * bits / 8))
+    # both operands in one launch (what Pipeline.Run does too); each on its own is
+    # timed after the steps, see `standalone` below
+    bytes_a, bytes_b = 2.0 * B * 2 * M * K * bits / 8, 2.0 * B * 2 * N * K * bits / 8
+    kernels.append(("transposes", lambda sa=a_cur, sb=b_cur: cc.Transpose.RunPair(
+        tr_a, sa.data_ptr(), a_t.data_ptr(), tr_b, sb.data_ptr(), b_t.data_ptr()), bytes_a + bytes_b))
+    standalone = [("transpose_a", lambda s=a_cur: tr_a.Run(s.data_ptr(), a_t.data_ptr()), bytes_a),
+                  ("transpose_b", lambda s=b_cur: tr_b.Run(s.data_ptr(), b_t.data_ptr()), bytes_b)]
     gemm = cc.GEMM(B, M, N, K, 0, stream, prec, cc.Variant.opt, AX.complex_planar, MO.row_major)
     run_gemm = lambda: gemm.Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
 
@@ -229,6 +232,24 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
         per_kernel[label + "_ms"] = ms
         per_kernel[label + "_gbs"] = nbytes / ms / 1e6
         per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
+
+    # The two transposes as separate launches, each 20 times back to back between
+    # two events (an event pair around a single 30 us launch adds some 4 us to it).
+    for label, fn, nbytes in standalone:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        e0.record()
+        for _ in range(20):
+            fn()
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1) / 20
+        per_kernel[label + "_ms"] = ms
+        per_kernel[label + "_gbs"] = nbytes / ms / 1e6
+        per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
+    per_kernel["method"] = ("gemm, transposes (both operands, one launch) and packing_*: event pairs "
+                            "inside the timed steps; transpose_a / transpose_b: separate launches, "
+                            "20 back to back between two events after the steps")
 
     if tin == VT.int1:
         dtype, peak, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "TOP/s"

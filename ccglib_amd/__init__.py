@@ -184,6 +184,14 @@ class Transpose(_Handle):
         _capi.check(_capi.load().ccglib_transpose_run_host(self._h, _ptr(h_input),
                                                           _ptr(d_output)))
 
+    @staticmethod
+    def RunPair(transpose_a, d_input_a, d_output_a, transpose_b, d_input_b, d_output_b):
+        """Both operands of one GEMM, in one kernel launch where they take the
+        same kernel (no counterpart in the reference)."""
+        _capi.check(_capi.load().ccglib_transpose_run_pair(
+            transpose_a._h, _ptr(d_input_a), _ptr(d_output_a),
+            transpose_b._h, _ptr(d_input_b), _ptr(d_output_b)))
+
 
 class Packing(_Handle):
     _destroy = "ccglib_packing_destroy"

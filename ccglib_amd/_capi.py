@@ -24,6 +24,7 @@ SIGNATURES = {
     "ccglib_transpose_create": (_i, [_pvp, _sz, _sz, _sz, _sz, _sz, _sz, _i, _vp, _i]),
     "ccglib_transpose_run": (_i, [_vp, _vp, _vp]),
     "ccglib_transpose_run_host": (_i, [_vp, _vp, _vp]),
+    "ccglib_transpose_run_pair": (_i, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "ccglib_transpose_destroy": (_i, [_vp]),
     "ccglib_packing_create": (_i, [_pvp, _sz, _i, _i, _vp, _i]),
     "ccglib_packing_run": (_i, [_vp, _vp, _vp]),

@@ -435,11 +435,11 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
     t.in = d_a;
     t.out = tiled_a;
     t.m = g->M;
-    hipError_t et = launch_transpose(t, g->stream);
-    t.in = d_b;
-    t.out = tiled_b;
-    t.m = g->N;
-    if (et == hipSuccess) et = launch_transpose(t, g->stream);
+    TransposeParams tb = t;
+    tb.in = d_b;
+    tb.out = tiled_b;
+    tb.m = g->N;
+    const hipError_t et = launch_transpose_pair(t, tb, g->stream);
     if (et != hipSuccess) return fail_hip(et, "re-tiling of ragged GEMM operands");
     fill_gemm_params(g, tiled_a, tiled_b, d_c, &p);
     p.variant = kOpt;
@@ -500,10 +500,8 @@ int ccglib_transpose_create(ccglib_transpose_t *transpose, size_t B, size_t M, s
   return CCGLIB_OK;
 }
 
-int ccglib_transpose_run(ccglib_transpose_t t, const void *d_input, void *d_output) {
-  if (!t) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null transpose handle");
-  if (t->B == 0 || t->M == 0 || t->N == 0) return CCGLIB_OK;
-  if (!d_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+static TransposeParams transpose_params(const ccglib_transpose *t, const void *d_input,
+                                        void *d_output) {
   TransposeParams p;
   p.in = d_input;
   p.out = d_output;
@@ -520,9 +518,41 @@ int ccglib_transpose_run(ccglib_transpose_t t, const void *d_input, void *d_outp
     p.n_chunk = t->N_chunk;
   }
   p.interleaved = (t->axis == kInterleaved);
+  return p;
+}
+
+int ccglib_transpose_run(ccglib_transpose_t t, const void *d_input, void *d_output) {
+  if (!t) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null transpose handle");
+  if (t->B == 0 || t->M == 0 || t->N == 0) return CCGLIB_OK;
+  if (!d_input || !d_output) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  const TransposeParams p = transpose_params(t, d_input, d_output);
   DeviceGuard guard(t->device);
   HIP_TRY(guard.status());
   const hipError_t e = launch_transpose(p, t->stream);
+  if (e != hipSuccess) return fail_hip(e, "transpose kernel launch");
+  return CCGLIB_OK;
+}
+
+int ccglib_transpose_run_pair(ccglib_transpose_t ta, const void *d_input_a, void *d_output_a,
+                              ccglib_transpose_t tb, const void *d_input_b, void *d_output_b) {
+  if (!ta || !tb) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null transpose handle");
+  if (ta->device != tb->device || ta->stream != tb->stream) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                "the two transposes of a pair must share their device and stream");
+  }
+  const bool empty_a = ta->B == 0 || ta->M == 0 || ta->N == 0;
+  const bool empty_b = tb->B == 0 || tb->M == 0 || tb->N == 0;
+  if (empty_a || empty_b) {
+    const int rc = empty_a ? CCGLIB_OK : ccglib_transpose_run(ta, d_input_a, d_output_a);
+    return rc != CCGLIB_OK || empty_b ? rc : ccglib_transpose_run(tb, d_input_b, d_output_b);
+  }
+  if (!d_input_a || !d_output_a || !d_input_b || !d_output_b) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null device pointer");
+  }
+  DeviceGuard guard(ta->device);
+  HIP_TRY(guard.status());
+  const hipError_t e = launch_transpose_pair(transpose_params(ta, d_input_a, d_output_a),
+                                             transpose_params(tb, d_input_b, d_output_b), ta->stream);
   if (e != hipSuccess) return fail_hip(e, "transpose kernel launch");
   return CCGLIB_OK;
 }
@@ -900,8 +930,9 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
     b = p->d_b_packed;
   }
   if (p->trans_a) {  // :116-121
-    if ((rc = ccglib_transpose_run(p->trans_a, a, p->d_a_trans))) return rc;
-    if ((rc = ccglib_transpose_run(p->trans_b, b, p->d_b_trans))) return rc;
+    if ((rc = ccglib_transpose_run_pair(p->trans_a, a, p->d_a_trans, p->trans_b, b, p->d_b_trans))) {
+      return rc;
+    }
     a = p->d_a_trans;
     b = p->d_b_trans;
   }
@@ -1190,11 +1221,11 @@ int ccglib_pipeline_run_static(size_t B, size_t M, size_t N, size_t K, int devic
   t.in = src_a;
   t.out = ws_a;
   t.m = M;
-  hipError_t e = launch_transpose(t, s);
-  t.in = src_b;
-  t.out = ws_b;
-  t.m = N;
-  if (e == hipSuccess) e = launch_transpose(t, s);
+  TransposeParams tb = t;
+  tb.in = src_b;
+  tb.out = ws_b;
+  tb.m = N;
+  hipError_t e = launch_transpose_pair(t, tb, s);
   if (e != hipSuccess) return fail_hip(e, "transpose kernel launch");
   GemmParams p;
   fill_gemm_params(&g, ws_a, ws_b, d_c, &p);

@@ -108,6 +108,10 @@ struct TransposeParams {
   int interleaved;
 };
 hipError_t launch_transpose(const TransposeParams &p, hipStream_t stream);
+// The two operands of one GEMM (rows of the same length): one launch where both
+// take the same kernel.
+hipError_t launch_transpose_pair(const TransposeParams &p0, const TransposeParams &p1,
+                                 hipStream_t stream);
 
 // Interleaved input may be `segments` buffers of n samples each, one after the
 // other, each packed on its own into ceil(n / 32) words (real bits, then

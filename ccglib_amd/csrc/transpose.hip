@@ -93,7 +93,7 @@ __device__ __forceinline__ void load_ragged(const char *p, size_t plane_stride_b
 
 constexpr int kRowsPerThread = 2;
 
-// grid: (ceil(n_vecs_padded / VPR), ceil(Mp / rows per block), B); block: 256
+// grid: (ceil(n_vecs_padded / VPR), ceil(Mp / rows per block) [of both operands], B); block: 256
 // threads as VPR vectors x 256 / VPR rows, each thread doing rows r and
 // r + 256 / VPR (two rows a thread measured best over the operand shapes of the
 // benchmark configurations: one row is as good for 16-bit but slower for 8-bit
@@ -103,12 +103,23 @@ constexpr int kRowsPerThread = 2;
 // 72 vectors: with 16 a tenth of the threads would idle).
 // RAGGED: input rows of any length at any element-aligned address (the output
 // tiles still hold whole vectors per row).
+// One launch can serve two operands with rows of the same length (the A and B
+// of one GEMM): block rows below y_split belong to the first, the others to
+// the second, which spares a small operand its own launch, ramp-up and tail.
+struct TransposePairArgs {
+  TransposeArgs op[2];
+  unsigned y_split;
+};
+
 template <int EB, bool INTERLEAVED, bool RAGGED, int VPR>
-__global__ __launch_bounds__(256) void transpose_vec(const TransposeArgs a) {
+__global__ __launch_bounds__(256) void transpose_vec(const TransposePairArgs pair) {
   constexpr int V = 16 / EB;  // elements per vector
   constexpr int RS = 256 / VPR;   // rows between the two rows of a thread
+  const bool second = blockIdx.y >= pair.y_split;
+  const TransposeArgs &a = pair.op[second ? 1 : 0];
   const size_t nvec = (size_t)blockIdx.x * VPR + (threadIdx.x % VPR);
-  const size_t m_base = (size_t)blockIdx.y * (RS * kRowsPerThread) + (threadIdx.x / VPR);
+  const size_t m_base = (size_t)(blockIdx.y - (second ? pair.y_split : 0u)) * (RS * kRowsPerThread) +
+                        (threadIdx.x / VPR);
   const size_t b = blockIdx.z;
   const size_t m_padded = a.m_tiles * a.m_chunk;
   if (nvec >= a.n_vecs_padded) return;
@@ -183,9 +194,16 @@ __global__ __launch_bounds__(256) void transpose_scalar(const TransposeArgs a, s
   out[o + plane] = im;
 }
 
-template <int EB, typename T>
-hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
+// What a launch of the vector kernel needs to know about one operand.
+template <int EB> struct VecPlan {
   TransposeArgs a;
+  bool out_vec_ok, in_vec_ok, narrow;
+  size_t y_blocks;
+};
+
+template <int EB> VecPlan<EB> plan_operand(const TransposeParams &p) {
+  VecPlan<EB> v;
+  TransposeArgs &a = v.a;
   a.in = static_cast<const char *>(p.in);
   a.out = static_cast<char *>(p.out);
   a.m = p.m;
@@ -196,48 +214,82 @@ hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
   a.n_tiles = ceil_div(p.n, p.n_chunk);
   constexpr size_t V = 16 / EB;
   const size_t m_padded = a.m_tiles * a.m_chunk, n_padded = a.n_tiles * a.n_chunk;
-  if (p.batch == 0 || m_padded == 0 || n_padded == 0) return hipSuccess;
   // whole vectors per output tile row; the input may be ragged
-  const bool narrow = (n_padded / V) % 16 != 0 && (n_padded / V) % 8 == 0;
-  const size_t vpr = narrow ? 8 : 16, rows_per_block = 256 / vpr * kRowsPerThread;
-  const bool out_vec_ok = (p.n_chunk % V == 0) && ((uintptr_t)p.out % 16 == 0) &&
-                          ((uintptr_t)p.in % EB == 0) && p.batch <= 65535 &&
-                          ceil_div(m_padded, rows_per_block) <= 65535;
-  const bool in_vec_ok = (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0);
-  if (out_vec_ok) {
-    a.n_vecs_padded = n_padded / V;
-    a.vecs_per_tile_row = p.n_chunk / V;
-    const dim3 grid((unsigned)ceil_div(a.n_vecs_padded, vpr),
-                    (unsigned)ceil_div(m_padded, rows_per_block), (unsigned)p.batch);
-    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, a); };
-    if (p.interleaved) {
-      if (in_vec_ok) {
-        narrow ? launch(transpose_vec<EB, true, false, 8>) : launch(transpose_vec<EB, true, false, 16>);
-      } else {
-        narrow ? launch(transpose_vec<EB, true, true, 8>) : launch(transpose_vec<EB, true, true, 16>);
-      }
+  v.narrow = (n_padded / V) % 16 != 0 && (n_padded / V) % 8 == 0;
+  const size_t rows_per_block = 256 / (v.narrow ? 8 : 16) * kRowsPerThread;
+  v.y_blocks = ceil_div(m_padded, rows_per_block);
+  v.out_vec_ok = (p.n_chunk % V == 0) && ((uintptr_t)p.out % 16 == 0) &&
+                 ((uintptr_t)p.in % EB == 0) && p.batch <= 65535 && v.y_blocks <= 65535;
+  v.in_vec_ok = (p.n % V == 0) && ((uintptr_t)p.in % 16 == 0);
+  a.n_vecs_padded = v.out_vec_ok ? n_padded / V : 0;
+  a.vecs_per_tile_row = v.out_vec_ok ? p.n_chunk / V : 0;
+  return v;
+}
+
+// p1 == nullptr: one operand. Otherwise the caller has checked that both take
+// the same kernel (same batch, row length, tile width, layout and raggedness).
+template <int EB>
+hipError_t launch_vec(const TransposeParams &p0, const VecPlan<EB> &v0, const VecPlan<EB> *v1,
+                      hipStream_t stream) {
+  TransposePairArgs pair;
+  pair.op[0] = v0.a;
+  pair.op[1] = v1 ? v1->a : v0.a;
+  pair.y_split = (unsigned)v0.y_blocks;
+  const size_t vpr = v0.narrow ? 8 : 16;
+  const dim3 grid((unsigned)ceil_div(v0.a.n_vecs_padded, vpr),
+                  (unsigned)(v0.y_blocks + (v1 ? v1->y_blocks : 0)), (unsigned)p0.batch);
+  auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, pair); };
+  const bool narrow = v0.narrow;
+  if (p0.interleaved) {
+    if (v0.in_vec_ok) {
+      narrow ? launch(transpose_vec<EB, true, false, 8>) : launch(transpose_vec<EB, true, false, 16>);
     } else {
-      if (in_vec_ok) {
-        narrow ? launch(transpose_vec<EB, false, false, 8>) : launch(transpose_vec<EB, false, false, 16>);
-      } else {
-        narrow ? launch(transpose_vec<EB, false, true, 8>) : launch(transpose_vec<EB, false, true, 16>);
-      }
+      narrow ? launch(transpose_vec<EB, true, true, 8>) : launch(transpose_vec<EB, true, true, 16>);
     }
   } else {
-    a.n_vecs_padded = 0;
-    a.vecs_per_tile_row = 0;
-    const size_t total = p.batch * m_padded * n_padded;
-    const size_t blocks = ceil_div(total, 256);
-    if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
-    if (p.interleaved) {
-      hipLaunchKernelGGL((transpose_scalar<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                         a, p.batch);
+    if (v0.in_vec_ok) {
+      narrow ? launch(transpose_vec<EB, false, false, 8>) : launch(transpose_vec<EB, false, false, 16>);
     } else {
-      hipLaunchKernelGGL((transpose_scalar<T, false>), dim3((unsigned)blocks), dim3(256), 0,
-                         stream, a, p.batch);
+      narrow ? launch(transpose_vec<EB, false, true, 8>) : launch(transpose_vec<EB, false, true, 16>);
     }
   }
   return hipGetLastError();
+}
+
+template <int EB, typename T>
+hipError_t launch_width(const TransposeParams &p, hipStream_t stream) {
+  const VecPlan<EB> v = plan_operand<EB>(p);
+  const TransposeArgs &a = v.a;
+  const size_t m_padded = a.m_tiles * a.m_chunk, n_padded = a.n_tiles * a.n_chunk;
+  if (p.batch == 0 || m_padded == 0 || n_padded == 0) return hipSuccess;
+  if (v.out_vec_ok) return launch_vec<EB>(p, v, nullptr, stream);
+  const size_t total = p.batch * m_padded * n_padded;
+  const size_t blocks = ceil_div(total, 256);
+  if (blocks > 0x7fffffffu) return hipErrorInvalidValue;
+  if (p.interleaved) {
+    hipLaunchKernelGGL((transpose_scalar<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, a,
+                       p.batch);
+  } else {
+    hipLaunchKernelGGL((transpose_scalar<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       a, p.batch);
+  }
+  return hipGetLastError();
+}
+
+template <int EB>
+bool try_launch_pair(const TransposeParams &p0, const TransposeParams &p1, hipStream_t stream,
+                     hipError_t &result) {
+  if (p0.batch != p1.batch || p0.n != p1.n || p0.n_chunk != p1.n_chunk ||
+      p0.interleaved != p1.interleaved || p0.batch == 0 || p0.n == 0 || p0.m == 0 || p1.m == 0) {
+    return false;
+  }
+  const VecPlan<EB> v0 = plan_operand<EB>(p0), v1 = plan_operand<EB>(p1);
+  if (!v0.out_vec_ok || !v1.out_vec_ok || v0.in_vec_ok != v1.in_vec_ok ||
+      v0.y_blocks + v1.y_blocks > 65535) {
+    return false;
+  }
+  result = launch_vec<EB>(p0, v0, &v1, stream);
+  return true;
 }
 
 }  // namespace
@@ -249,6 +301,25 @@ hipError_t launch_transpose(const TransposeParams &p, hipStream_t stream) {
     case 4: return launch_width<4, unsigned>(p, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+// Both operands of one GEMM. One launch when they take the same vector kernel,
+// otherwise one launch each.
+hipError_t launch_transpose_pair(const TransposeParams &p0, const TransposeParams &p1,
+                                 hipStream_t stream) {
+  hipError_t e = hipSuccess;
+  bool done = false;
+  if (p0.elem_bytes == p1.elem_bytes) {
+    switch (p0.elem_bytes) {
+      case 1: done = try_launch_pair<1>(p0, p1, stream, e); break;
+      case 2: done = try_launch_pair<2>(p0, p1, stream, e); break;
+      case 4: done = try_launch_pair<4>(p0, p1, stream, e); break;
+      default: return hipErrorInvalidValue;
+    }
+  }
+  if (done) return e;
+  e = launch_transpose(p0, stream);
+  return e == hipSuccess ? launch_transpose(p1, stream) : e;
 }
 
 }  // namespace ccglib_amd

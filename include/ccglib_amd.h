@@ -157,6 +157,17 @@ CCGLIB_API int ccglib_transpose_run(ccglib_transpose_t transpose,
                                     const void *d_input, void *d_output);
 CCGLIB_API int ccglib_transpose_run_host(ccglib_transpose_t transpose,
                                          const void *h_input, void *d_output);
+/* Both operands of one GEMM: the same as ccglib_transpose_run on each, in one
+ * kernel launch where the two have the same batch size, row length N, N_chunk,
+ * width and input layout (otherwise in two). No counterpart in the reference,
+ * whose pipeline launches one transpose per operand
+ * (src/pipeline/Pipeline.cpp:116-121); a small operand no longer pays for a
+ * launch, ramp-up and tail of its own. Both objects must have been created
+ * for the same device and stream. */
+CCGLIB_API int ccglib_transpose_run_pair(ccglib_transpose_t transpose_a,
+                                         const void *d_input_a, void *d_output_a,
+                                         ccglib_transpose_t transpose_b,
+                                         const void *d_input_b, void *d_output_b);
 CCGLIB_API int ccglib_transpose_destroy(ccglib_transpose_t transpose);
 
 /* ------------------------------------------------------------------------

@@ -80,3 +80,53 @@ def test_host_input():
 def test_empty():
     t = cc.Transpose(0, 16, 16, 16, 16, 16, 0, stream())
     t.Run(0, 0)
+
+
+@pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
+@pytest.mark.parametrize("bits,kc,Ma,Mb,N,Mca,Mcb,skew", [
+    (16, 32, 512, 4096, 576, 128, 128, 0),    # beamformer operands: rows of 72 vectors
+    (16, 32, 100, 300, 1000, 128, 64, 0),     # ragged rows and columns, different row tiles
+    (8, 64, 77, 130, 257, 128, 128, 0),       # rows that are not whole vectors
+    (32, 16, 64, 200, 96, 128, 128, 0),
+    (16, 32, 129, 64, 264, 128, 128, 1),      # first operand not 16-byte aligned: two launches
+    (1, 512, 100, 256, 1056, 128, 128, 0),    # 1-bit words
+    (16, 32, 5, 7, 7, 128, 128, 0),           # scalar kernel for both
+])
+def test_pair_matches_oracle(axis, bits, kc, Ma, Mb, N, Mca, Mcb, skew):
+    """ccglib_transpose_run_pair: both operands as the oracle transposes each."""
+    B = 3
+    rng = np.random.default_rng(Ma + Mb + N)
+    dt = NP[bits]
+    nw = N // 32 if bits == 1 else N
+    outs, args, keep = [], [], []
+    for M, Mc, sk in ((Ma, Mca, skew), (Mb, Mcb, 0)):
+        x = rng.integers(1, np.iinfo(dt).max, B * 2 * M * nw, dtype=dt, endpoint=True)
+        want = orc.transpose(x, B, M, N, Mc, kc, bits, int(axis))
+        d_out = to_device(np.full(want.size, 0xA5, dtype=dt))
+        d_in = to_device(np.concatenate([np.zeros(sk, dtype=dt), x]))
+        t = cc.Transpose(B, M, N, Mc, kc, bits, 0, stream(), axis)
+        keep.append((d_in, t))
+        args += [t, d_in.data_ptr() + sk * dt().itemsize, d_out.data_ptr()]
+        outs.append((d_out, want))
+    cc.Transpose.RunPair(*args)
+    torch.cuda.synchronize()
+    for d_out, want in outs:
+        assert np.array_equal(to_host(d_out, dt), want)
+
+
+def test_pair_of_different_rows_falls_back():
+    """Operands whose rows differ in length cannot share a launch: still both done."""
+    rng = np.random.default_rng(5)
+    outs, args, keep = [], [], []
+    for M, N in ((64, 128), (32, 256)):
+        x = rng.integers(1, 65535, 2 * 2 * M * N, dtype=np.uint16, endpoint=True)
+        want = orc.transpose(x, 2, M, N, 64, 32, 16, int(PLANAR))
+        d_out, d_in = to_device(np.zeros(want.size, dtype=np.uint16)), to_device(x)
+        t = cc.Transpose(2, M, N, 64, 32, 16, 0, stream(), PLANAR)
+        keep.append((d_in, t))
+        args += [t, d_in.data_ptr(), d_out.data_ptr()]
+        outs.append((d_out, want))
+    cc.Transpose.RunPair(*args)
+    torch.cuda.synchronize()
+    for d_out, want in outs:
+        assert np.array_equal(to_host(d_out, np.uint16), want)
