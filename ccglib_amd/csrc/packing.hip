@@ -84,42 +84,40 @@ __global__ __launch_bounds__(256) void pack_planar_vec(const unsigned char *__re
 template <bool ALIGNED>
 __global__ __launch_bounds__(256) void pack_interleaved_vec(const unsigned char *__restrict__ in,
                                                             unsigned *__restrict__ out,
-                                                            size_t seg16, size_t segments) {
-  const size_t n16 = seg16 * segments;
+                                                            size_t seg16) {
+  // blockIdx.y: the segment (no division per item to find it)
+  const size_t seg_words = seg16 / 2;        // packed words of one segment
+  in += (size_t)blockIdx.y * seg16 * 16;
+  unsigned *o_re = out + (size_t)blockIdx.y * seg_words, *o_im = o_re + seg_words / 2;
   const size_t stride = (size_t)gridDim.x * 256 * kPackPerThread;
   const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const size_t seg_words = seg16 / 2;        // packed words of one segment
-  for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kPackPerThread; base < n16; base += stride) {
+  for (size_t base = ((size_t)blockIdx.x * 4 + wave) * 64 * kPackPerThread; base < seg16; base += stride) {
     uint4_t v[kPackPerThread];
 #pragma unroll
     for (int k = 0; k < kPackPerThread; ++k) {
       const size_t gi = base + k * 64 + lane;
-      v[k] = gi < n16 ? load16<ALIGNED>(in + gi * 16) : uint4_t{0, 0, 0, 0};
+      v[k] = gi < seg16 ? load16<ALIGNED>(in + gi * 16) : uint4_t{0, 0, 0, 0};
     }
 #pragma unroll
     for (int k = 0; k < kPackPerThread; ++k) {
       const size_t gi = base + k * 64 + lane;
-      const unsigned b = bits_of16(v[k]);  // bit 2p = re of pair p, bit 2p+1 = im
-      // gather even bits into the low byte, odd bits into the second byte
-      unsigned e = b & 0x5555u, o = (b >> 1) & 0x5555u;
-      e = (e | (e >> 1)) & 0x3333u;
-      e = (e | (e >> 2)) & 0x0f0fu;
-      e = (e | (e >> 4)) & 0x00ffu;
-      o = (o | (o >> 1)) & 0x3333u;
-      o = (o | (o >> 2)) & 0x0f0fu;
-      o = (o | (o >> 4)) & 0x00ffu;
-      const unsigned mine = e | (o << 8);
+      // real parts are the even bytes, imaginary parts the odd ones: gather each
+      // kind into two words first, then 4 bytes -> 4 bits as in the planar kernel
+      const unsigned re_lo = __builtin_amdgcn_perm(v[k][1], v[k][0], 0x06040200u);
+      const unsigned re_hi = __builtin_amdgcn_perm(v[k][3], v[k][2], 0x06040200u);
+      const unsigned im_lo = __builtin_amdgcn_perm(v[k][1], v[k][0], 0x07050301u);
+      const unsigned im_hi = __builtin_amdgcn_perm(v[k][3], v[k][2], 0x07050301u);
+      const unsigned mine = nibble_of(re_lo) | (nibble_of(re_hi) << 4) | (nibble_of(im_lo) << 8) |
+                            (nibble_of(im_hi) << 12);
       const unsigned l1 = __shfl_down(mine, 1), l2 = __shfl_down(mine, 2),
                      l3 = __shfl_down(mine, 3);
-      if ((lane & 3) == 0 && gi < n16) {
+      if ((lane & 3) == 0 && gi < seg16) {
         const unsigned re = (mine & 0xffu) | ((l1 & 0xffu) << 8) | ((l2 & 0xffu) << 16) |
                             ((l3 & 0xffu) << 24);
         const unsigned im = ((mine >> 8) & 0xffu) | (((l1 >> 8) & 0xffu) << 8) |
                             (((l2 >> 8) & 0xffu) << 16) | (((l3 >> 8) & 0xffu) << 24);
-        const size_t seg = gi / seg16, local = gi % seg16;
-        unsigned *o_seg = out + seg * seg_words;
-        o_seg[local >> 2] = re;
-        o_seg[seg_words / 2 + (local >> 2)] = im;
+        o_re[gi >> 2] = re;
+        o_im[gi >> 2] = im;
       }
     }
   }
@@ -232,11 +230,17 @@ hipError_t launch_pack_bits(const unsigned char *in, unsigned *out, size_t n, in
   } else if (n % 64 == 0) {
     vec_words = words;
     const size_t seg16 = n / 16;
-    const dim3 grid(grid_for(seg16 * segments, kPackPerThread));
-    if (aligned) {
-      hipLaunchKernelGGL(pack_interleaved_vec<true>, grid, dim3(256), 0, stream, in, out, seg16, segments);
-    } else {
-      hipLaunchKernelGGL(pack_interleaved_vec<false>, grid, dim3(256), 0, stream, in, out, seg16, segments);
+    // one grid row per segment, at most 65535 rows a launch
+    for (size_t first = 0; first < segments; first += 65535) {
+      const size_t rows = segments - first < 65535 ? segments - first : 65535;
+      const dim3 grid(grid_for(seg16, kPackPerThread), (unsigned)rows);
+      const unsigned char *src = in + first * n;
+      unsigned *dst = out + first * seg_words;
+      if (aligned) {
+        hipLaunchKernelGGL(pack_interleaved_vec<true>, grid, dim3(256), 0, stream, src, dst, seg16);
+      } else {
+        hipLaunchKernelGGL(pack_interleaved_vec<false>, grid, dim3(256), 0, stream, src, dst, seg16);
+      }
     }
   }
   if (vec_words < words) {
