@@ -117,6 +117,15 @@ static void test_opt_with_transpose(hipDevice_t device, hipStream_t stream) {
              got[((bb * 2 + 1) * M + m) * N + n] == want.imag();
       }
   CHECK(ok);
+  // and against the host-side class, batch by batch, as the reference's tests
+  // verify (test/gemm/verify.h:54-60)
+  ccglib::reference::GEMM host;
+  std::vector<float> want_host = hc;
+  for (size_t bb = 0; bb < B; ++bb) {
+    host.Run(ha.data() + bb * 2 * M * K, hb.data() + bb * 2 * N * K, want_host.data() + bb * 2 * M * N,
+             M, N, K, ccglib::mma::row_major, alpha, beta);
+  }
+  CHECK(want_host == got);
 }
 
 // pack, unpack and the round trip on N = 2048 (test/hip/packing.cpp)
