@@ -241,14 +241,21 @@ __device__ __forceinline__ void mma_step(const char *const (&slot)[DtypeTraits<D
 // of the MFMA are exchanged (Y supplies the instruction's "A" rows, X its "B"
 // columns), which transposes what a lane holds of every 16 x 16 tile.
 // FIRST: the first K tile of a C tile; the sums start from zero.
-template <int DT, int BX, int BY, bool XT, bool FIRST, typename Mid>
-__device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&xo)[4], int y_frag_off,
+// xa[i] / ya: the lane's LDS address of the X fragment of tile i / of the Y
+// fragment of tile row 0 in the current slots. late(): called among the MFMAs
+// of the last tile row, for whatever the next iteration needs computed (its
+// addresses, the slot numbers): work placed there is hidden behind MFMAs, work
+// left between the last MFMA and the barrier is not.
+template <int DT, int BX, int BY, bool XT, bool FIRST, typename Mid, typename Late>
+__device__ __forceinline__ void mma_step_ordered(const unsigned (&xa)[4], unsigned ya,
                                                  float4_t (&acc_re)[4][4], float4_t (&acc_im)[4][4],
-                                                 Mid &&mid) {
+                                                 Mid &&mid, Late &&late) {
   static_assert(DtypeTraits<DT>::kTilesPerMfma == 1, "one K tile per MFMA");
-  auto rd = [&](int off) {
+  // (LDS addresses as 32-bit numbers: the read's address register is the number itself)
+  typedef __attribute__((address_space(3))) const int4_t lds_int4_t;
+  auto rd = [](unsigned address) {
     Fragment<DT> f;
-    f.v[0] = *reinterpret_cast<const int4_t *>(slot + off);
+    f.v[0] = *reinterpret_cast<lds_int4_t *>(address);
     return f;
   };
   auto mm = [](const Fragment<DT> &x, const Fragment<DT> &y, float4_t acc) {
@@ -258,37 +265,37 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&x
   constexpr int ROW16 = 16 * kTileRowBytes, XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;
 #define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
   Fragment<DT> xr[4], xi[4], yr, yi, yin, yr_next, yi_next;
-  yr = rd(y_frag_off);
-  xr[0] = rd(xo[0]);
-  xr[1] = rd(xo[1]);
-  xr[2] = rd(xo[2]);
+  yr = rd(ya);
+  xr[0] = rd(xa[0]);
+  xr[1] = rd(xa[1]);
+  xr[2] = rd(xa[2]);
   CCGLIB_PIN;
   acc_re[0][0] = mm(xr[0], yr, c0(acc_re[0][0]));
-  xr[3] = rd(xo[3]);
+  xr[3] = rd(xa[3]);
   CCGLIB_PIN;
   acc_re[0][1] = mm(xr[1], yr, c0(acc_re[0][1]));
-  yi = rd(y_frag_off + YP);
+  yi = rd(ya + YP);
   CCGLIB_PIN;
   acc_re[0][2] = mm(xr[2], yr, c0(acc_re[0][2]));
-  xi[0] = rd(xo[0] + XP);
+  xi[0] = rd(xa[0] + XP);
   CCGLIB_PIN;
   acc_re[0][3] = mm(xr[3], yr, c0(acc_re[0][3]));
-  xi[1] = rd(xo[1] + XP);
+  xi[1] = rd(xa[1] + XP);
   CCGLIB_PIN;
   acc_im[0][0] = mm(xr[0], yi, c0(acc_im[0][0]));
-  xi[2] = rd(xo[2] + XP);
+  xi[2] = rd(xa[2] + XP);
   CCGLIB_PIN;
   acc_im[0][1] = mm(xr[1], yi, c0(acc_im[0][1]));
-  xi[3] = rd(xo[3] + XP);
+  xi[3] = rd(xa[3] + XP);
   CCGLIB_PIN;
   acc_im[0][2] = mm(xr[2], yi, c0(acc_im[0][2]));
   yin = negate<DT>(yi);
   CCGLIB_PIN;
   acc_im[0][3] = mm(xr[3], yi, c0(acc_im[0][3]));
-  yr_next = rd(y_frag_off + ROW16);
+  yr_next = rd(ya + ROW16);
   CCGLIB_PIN;
   acc_re[0][0] = mm(xi[0], yin, acc_re[0][0]);
-  yi_next = rd(y_frag_off + YP + ROW16);
+  yi_next = rd(ya + YP + ROW16);
   CCGLIB_PIN;
   acc_im[0][0] = mm(xi[0], yr, acc_im[0][0]);
 #pragma unroll
@@ -312,14 +319,18 @@ __device__ __forceinline__ void mma_step_ordered(const char *slot, const int (&x
     acc_im[j][0] = mm(xr[0], yi, c0(acc_im[j][0]));
     acc_im[j][1] = mm(xr[1], yi, c0(acc_im[j][1]));
     acc_re[j][1] = mm(xr[1], yr, c0(acc_re[j][1]));
-    if (j < 3) yr_next = rd(y_frag_off + (j + 1) * ROW16);
+    if (j < 3) yr_next = rd(ya + (j + 1) * ROW16);
     CCGLIB_PIN;
     acc_re[j][2] = mm(xr[2], yr, c0(acc_re[j][2]));
     acc_im[j][2] = mm(xr[2], yi, c0(acc_im[j][2]));
     acc_im[j][3] = mm(xr[3], yi, c0(acc_im[j][3]));
     acc_re[j][3] = mm(xr[3], yr, c0(acc_re[j][3]));
-    if (j < 3) yi_next = rd(y_frag_off + YP + (j + 1) * ROW16);
+    if (j < 3) yi_next = rd(ya + YP + (j + 1) * ROW16);
     CCGLIB_PIN;
+    if (j == 3) {
+      late();
+      CCGLIB_PIN;
+    }
     acc_im[j][0] = mm(xi[0], yr, acc_im[j][0]);
     acc_re[j][0] = mm(xi[0], yin, acc_re[j][0]);
     acc_re[j][1] = mm(xi[1], yin, acc_re[j][1]);
@@ -1674,6 +1685,10 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
     issue_x(t + XLEAD);
   }
   unsigned x_slot = 0, y_slot = 0;         // slots of the current iteration
+  // (hand-ordered 16-row step) the lane's fragment addresses in the current slots
+  unsigned xa[4], ya = lds_base + y_slot_off(0) + (y_frag_off - X_BYTES);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) xa[i] = lds_base + x_slot_off(0) + xo[i];
   const unsigned iters = k_tiles;
   for (unsigned vt = blockIdx.x; vt < total; vt += gridDim.x) {
     typename AccType<MS>::type acc_re[TY][TX], acc_im[TY][TX];
@@ -1702,56 +1717,67 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
       } else {
         wait_vmcnt_then_barrier<kOutstandingOk>();
       }
-      // the slots of the previous iteration are free now: refill them with the
-      // K tiles that are XLEAD / YLEAD iterations ahead (of this C tile or the next)
-      unsigned x_refill = x_slot + XLEAD, y_refill = y_slot + YLEAD;
-      x_refill = x_refill >= XSLOTS ? x_refill - XSLOTS : x_refill;
-      y_refill = y_refill >= SLOTS ? y_refill - SLOTS : y_refill;
-      // The copy instructions go out after the first group of MFMAs: right
+      // The slots of the previous iteration are free now: refill them with the
+      // K tiles that are XLEAD / YLEAD iterations ahead (of this C tile or the
+      // next). The copy instructions go out after the first group of MFMAs: right
       // after the barrier every wave of the block would otherwise be busy with
       // their address arithmetic and the matrix cores would have nothing to do.
       auto refill_slots = [&] {
+        unsigned x_refill = x_slot + XLEAD, y_refill = y_slot + YLEAD;
+        x_refill = x_refill >= XSLOTS ? x_refill - XSLOTS : x_refill;
+        y_refill = y_refill >= SLOTS ? y_refill - SLOTS : y_refill;
         issue_y(y_refill);
         issue_x(x_refill);
       };
-      const char *slot_ptr = lds + x_slot_off(x_slot);
-      // (the fragment offsets of Y count from the start of an [X | Y] slot)
-      const int y_shift = (int)y_slot_off(y_slot) - (int)x_slot_off(x_slot) - X_BYTES;
-      if constexpr (IL && MS == 32) {
-        static_assert(TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
-        mma_step32_interleaved<DT, BX, BY>(slot_ptr, xil32_off, yil32_off, acc_re, acc_im,
-                                           refill_slots);
-      } else if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
-        mma_step_interleaved_ordered<DT, BX, BY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
-                                                 refill_slots);
-      } else if constexpr (IL) {
-        mma_step_interleaved<DT, BX, BY, TX, TY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
-                                                 refill_slots);
-      } else {
-        const char *tile[KPM] = {slot_ptr};
-        if constexpr (DT == kInt1) {
-          static_assert(MS == 32 && TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
-          mma_step32_bits<BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
-        } else if constexpr (MS == 32 && TX == 2 && TY == 2) {
-          mma_step32_ordered<DT, BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
-        } else if constexpr (MS == 32) {
-          mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
-        } else if constexpr (TX == 4 && TY == 4) {
-          // (the first iteration of a C tile starts its sums from zero instead of
-          // from accumulators that would have to be cleared first)
-          if (it == 0) {
-            mma_step_ordered<DT, BX, BY, XT, true>(tile[0], xo, y_frag_off + y_shift, acc_re, acc_im,
-                                                   refill_slots);
-          } else {
-            mma_step_ordered<DT, BX, BY, XT, false>(tile[0], xo, y_frag_off + y_shift, acc_re, acc_im,
-                                                    refill_slots);
-          }
+      const unsigned x_next = x_slot + 1 == XSLOTS ? 0 : x_slot + 1;
+      const unsigned y_next = y_slot + 1 == SLOTS ? 0 : y_slot + 1;
+      if constexpr (kStepClears) {
+        // (the first iteration of a C tile starts its sums from zero instead of
+        // from accumulators that would have to be cleared first; the fragment
+        // addresses of the next iteration are worked out among the last MFMAs
+        // of this one, so that only the wait and the barrier stand between two
+        // iterations' MFMAs)
+        // (no fragment is read after the step calls this, so it overwrites in place)
+        auto next_addresses = [&] {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xa[i] = lds_base + x_slot_off(x_next) + xo[i];
+          ya = lds_base + y_slot_off(y_next) + (y_frag_off - X_BYTES);
+        };
+        if (it == 0) {
+          mma_step_ordered<DT, BX, BY, XT, true>(xa, ya, acc_re, acc_im, refill_slots,
+                                                 next_addresses);
         } else {
-          mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
+          mma_step_ordered<DT, BX, BY, XT, false>(xa, ya, acc_re, acc_im, refill_slots,
+                                                  next_addresses);
+        }
+      } else {
+        const char *slot_ptr = lds + x_slot_off(x_slot);
+        if constexpr (IL && MS == 32) {
+          static_assert(TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
+          mma_step32_interleaved<DT, BX, BY>(slot_ptr, xil32_off, yil32_off, acc_re, acc_im,
+                                             refill_slots);
+        } else if constexpr (IL && DtypeTraits<DT>::kElemBytes == 2 && TX == 4 && TY == 4) {
+          mma_step_interleaved_ordered<DT, BX, BY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
+                                                   refill_slots);
+        } else if constexpr (IL) {
+          mma_step_interleaved<DT, BX, BY, TX, TY>(slot_ptr, xil_off, yil_off, acc_re, acc_im,
+                                                   refill_slots);
+        } else {
+          const char *tile[KPM] = {slot_ptr};
+          if constexpr (DT == kInt1) {
+            static_assert(MS == 32 && TX == 2 && TY == 2, "2 x 2 tiles of 32 x 32 per wave");
+            mma_step32_bits<BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+          } else if constexpr (MS == 32 && TX == 2 && TY == 2) {
+            mma_step32_ordered<DT, BX, BY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+          } else if constexpr (MS == 32) {
+            mma_step32<DT, BX, BY, TX, TY>(tile[0], x32_off, y32_off, acc_re, acc_im, refill_slots);
+          } else {
+            mma_step<DT, BX, BY, TX, TY>(tile, x_frag_off, y_frag_off, acc_re, acc_im, refill_slots);
+          }
         }
       }
-      x_slot = x_slot + 1 == XSLOTS ? 0 : x_slot + 1;
-      y_slot = y_slot + 1 == SLOTS ? 0 : y_slot + 1;
+      x_slot = x_next;
+      y_slot = y_next;
     }
     // The stores below are not waited for here: they drain while the next C
     // tile is being computed. The counter cannot tell loads from stores, so
