@@ -164,7 +164,14 @@ int main(int argc, char **argv) {
     CHECK(hipEventElapsedTime(&best, e0, e1));
     best /= iters;
     const double tflops = 8.0 * B * M * N * K / (best * 1e-3) / 1e12;
-    std::printf("%-40s %10.4f %12.1f %9.1f%%\n", c.name, best, tflops, 100 * tflops / peak_of(c.type_in));
+    // a hash of C's bits: configurations that multiply the same operands in the same
+    // layout with the same MFMA shape must agree
+    std::vector<unsigned> hc(c_bytes / 4);
+    CHECK(hipMemcpy(hc.data(), dc, c_bytes, hipMemcpyDeviceToHost));
+    unsigned long long hash = 1469598103934665603ull;
+    for (unsigned v : hc) hash = (hash ^ v) * 1099511628211ull;
+    std::printf("%-40s %10.4f %12.1f %9.1f%%   C %016llx\n", c.name, best, tflops,
+                100 * tflops / peak_of(c.type_in), hash);
     std::fflush(stdout);
     CHECK(hipFree(dx));
     CHECK(hipFree(dy));
