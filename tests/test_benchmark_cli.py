@@ -94,9 +94,18 @@ def test_tuner_sweeps_its_configurations():
     for want in ("f16 256x128 w64x64 s3 m16 xt", "fp8 256x128 w64x64 s3 m32", "int1 256x128 w64x64 s3 m32",
                  "f16 planar 256x128 w64x64 s3 m16 xt", "f16 interleaved 256x128 w64x64 s3 m16"):
         assert want in names, want
+    hashes = {}
     for l in rows:
-        ms, rate = float(l.split()[-3]), float(l.split()[-2])
+        # "<name>  <ms>  <rate>  <percent>%   C <hash of C's bits>"
+        fields = l.split()
+        assert fields[-2] == "C" and fields[-3].endswith("%")
+        ms, rate = float(fields[-5]), float(fields[-4])
         assert ms > 0 and rate > 0
+        hashes[" ".join(fields[:-5])] = fields[-1]
+    # the same operands, layout and MFMA shape: the same bits, whatever the block shape,
+    # the epilogue or the ring
+    assert hashes["f16 256x128 w64x64 s3 m16 xt"] == hashes["f16 128x256 w64x64 s3 m16 xt"]
+    assert hashes["f16 256x128 w64x64 s3 m16 xt"] == hashes["f16 128x256 w64x64 y3 x4 m16 xt"]
     # a filter selects configurations by name
     r = subprocess.run([TUNE, "2", "256", "256", "64", "bf16"], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and all("bf16" in l for l in r.stdout.strip().splitlines()[1:])
