@@ -118,6 +118,12 @@ CCGLIB_API int ccglib_amd_get_option(int option, size_t *value);
  * 1-bit input: K must be a multiple of 32; alpha and beta are truncated to
  * integers (src/reference/GEMM.cpp:202-205).
  * C is read only when beta != 0.
+ * K whose interleaved row (2 * K * bits / 8 bytes) does not fit 32 bits is
+ * refused. Operands should be 16-byte aligned: basic-variant operands that are
+ * not (or whose rows are not whole 16-byte chunks) are re-tiled into a
+ * workspace the object owns (allocated at creation for such K, at the first
+ * such Run for such pointers; see CCGLIB_AMD_OPTION_BASIC_RETILE); opt-variant
+ * operands that are not are refused by Run.
  * ---------------------------------------------------------------------- */
 CCGLIB_API int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M,
                                   size_t N, size_t K, int device, void *stream,
@@ -196,8 +202,15 @@ CCGLIB_API int ccglib_packing_destroy(ccglib_packing_t packing);
  * include/ccglib/pipeline/pipeline.h:44-53 (src/pipeline/Pipeline.cpp:145-160),
  * Run(device) :54 (src/pipeline/Pipeline.cpp:183-188), Run(host) :41
  * (src/pipeline/Pipeline.cpp:162-176).
- * 1-bit input is one byte per sample and is packed first; the opt variant
- * transposes A and B first. Argument order follows the reference constructor.
+ * 1-bit input is one byte per sample and is packed first (interleaved input:
+ * every batch on its own, real bits then imaginary bits, which needs M*K and
+ * N*K to be multiples of 32 when B > 1; the reference packs the whole buffer
+ * as one, kernels/packing_kernel.cu:15-22, which is the same for B = 1); the
+ * opt variant transposes A and B first. 8- and 16-bit interleaved input whose
+ * rows are whole 16-byte chunks is read by the GEMM in place instead (no
+ * transposes); if a Run then gets pointers that are not 16-byte aligned, the
+ * object builds the pipeline with transposes at that Run and uses it for such
+ * calls. Argument order follows the reference constructor.
  * run_host copies a, b (and c when beta != 0) to the device, runs, copies c
  * back and returns when c is complete; sizes are those of the layouts above.
  * Jobs of 8 MiB or more with several batches move in chunks of whole batches
