@@ -82,6 +82,8 @@ def test_null_handles_are_errors_not_crashes():
     assert lib.ccglib_gemm_run(None, None, None, None) != 0
     assert b"null" in lib.ccglib_last_error()
     assert lib.ccglib_transpose_run(None, None, None) != 0
+    assert lib.ccglib_transpose_run_pair(None, None, None, None, None, None) != 0
+    assert b"null" in lib.ccglib_last_error()
     assert lib.ccglib_packing_run(None, None, None) != 0
     assert lib.ccglib_pipeline_run(None, None, None, None) != 0
     assert lib.ccglib_gemm_destroy(None) == 0
