@@ -877,10 +877,22 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
         Tout *pr = cbase + (size_t)y * nx + x;
         Tout *pi = pr + (size_t)nx * ny;
         if (have_beta) {
+          // (whole pieces: C comes in with one wide load per plane)
+          Tout cr4[4], ci4[4];
+          if (full) {
+            typedef Tout Piece __attribute__((ext_vector_type(4)));
+            const Piece vr = *reinterpret_cast<const Piece *>(pr), vi = *reinterpret_cast<const Piece *>(pi);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              cr4[e] = vr[e];
+              ci4[e] = vi[e];
+            }
+          }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if (x + e < nx) {
-              const float cr = (float)pr[e], ci = (float)pi[e];
+            if (full || x + e < nx) {
+              const float cr = full ? (float)cr4[e] : (float)pr[e];
+              const float ci = full ? (float)ci4[e] : (float)pi[e];
               re[e] += br * cr - bi * ci;
               im[e] += bi * cr + br * ci;
             }
@@ -908,10 +920,18 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
       } else {
         Tout *p = cbase + ((size_t)y * nx + x) * 2;
         if (have_beta) {
+          Tout c8[8];
+          if (full) {
+            typedef Tout Piece __attribute__((ext_vector_type(8)));
+            const Piece v = *reinterpret_cast<const Piece *>(p);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) c8[e] = v[e];
+          }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if (x + e < nx) {
-              const float cr = (float)p[2 * e], ci = (float)p[2 * e + 1];
+            if (full || x + e < nx) {
+              const float cr = full ? (float)c8[2 * e] : (float)p[2 * e];
+              const float ci = full ? (float)c8[2 * e + 1] : (float)p[2 * e + 1];
               re[e] += br * cr - bi * ci;
               im[e] += bi * cr + br * ci;
             }
