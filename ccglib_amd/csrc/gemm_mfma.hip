@@ -1975,7 +1975,16 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   }
   if (p.variant == kOpt || planar_direct) {
     if constexpr (KPM == 1) {
-      // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring
+      // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring.
+      // Interleaved fp32 C: in the exchanged-roles layout a lane's (re, im) pairs of
+      // a row lie 32 bytes apart, so every store instruction would write half
+      // cache lines; the other layout regroups the tile through LDS into whole
+      // rows of pairs (measured 5 % faster at B=64 512x4096x576).
+      if constexpr (TOUT == kFloat32) {
+        if (p.variant == kOpt && p.c_interleaved) {
+          return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, false>(p, stream);
+        }
+      }
       return p.variant == kOpt
                  ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>(p, stream)
                  : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>(p, stream);
