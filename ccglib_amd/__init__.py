@@ -92,6 +92,7 @@ class Option(enum.IntEnum):
     int1_popcount = 0
     basic_retile = 1
     host_chunk_bytes = 2
+    gemm_block_tile = 3
 
 
 def set_option(option, value):

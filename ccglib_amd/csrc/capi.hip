@@ -119,6 +119,7 @@ struct ccglib_gemm {
   // 1-bit GEMM: the MFMA kernel multiplies the packed words (0: the option that
   // keeps it on the vector ALUs was set when the object was created)
   int int1_direct = 1;
+  int block_tile = 0;
 };
 
 struct ccglib_transpose {
@@ -177,7 +178,7 @@ struct ccglib_pipeline {
 namespace {
 
 // Process-wide options (ccglib_amd_set_option), read when an object is created.
-size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0};
+size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0, 0};
 
 // Largest buffer of 1-bit tiles a pipeline allocates; beyond it the pipeline
 // runs the reference's sequence of kernels on its packed / transposed buffers.
@@ -249,6 +250,7 @@ void fill_gemm_params(const ccglib_gemm *g, const void *d_a, const void *d_b, vo
   p.workspace = g->workspace;
   p.workspace_bytes = g->workspace_bytes;
   p.int1_direct = g->int1_direct;
+  p.block_tile = g->block_tile;
 }
 
 }  // namespace
@@ -325,6 +327,9 @@ int ccglib_amd_set_option(int option, size_t value) {
   if (option < 0 || option >= CCGLIB_AMD_OPTION_COUNT) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "unknown option %d", option);
   }
+  if (option == CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE && value > 2) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "GEMM_BLOCK_TILE is 0, 1 or 2 (got %zu)", value);
+  }
   g_options[option] = value;
   return CCGLIB_OK;
 }
@@ -375,6 +380,7 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
             c_mem_order, alpha_re, alpha_im, beta_re, beta_im);
   g->retile_allowed = g_options[CCGLIB_AMD_OPTION_BASIC_RETILE] != 0;
   g->int1_direct = g_options[CCGLIB_AMD_OPTION_INT1_POPCOUNT] == 0;
+  g->block_tile = (int)g_options[CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE];
   // Planar rows that direct-to-LDS copies cannot fetch in whole chunks (for 1-bit
   // input: rows of K / 32 words). Re-tiling them costs two bandwidth-bound passes
   // and a copy of A and B; the kernel for the tiled layout then runs several

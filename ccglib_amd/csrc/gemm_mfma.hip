@@ -1954,6 +1954,22 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Whether 128 x 128 block tiles beat 256 x 128 ones for this problem: they do
+// when the larger tiles would leave compute units without work (fewer tiles
+// than units, or a last round that is mostly empty), although the smaller
+// block moves a third more bytes from L2 to LDS per flop (`penalty`: how much
+// slower per flop it measured once every unit is busy). Estimated from the
+// fraction of unit-rounds that hold a tile under either tiling.
+inline bool small_tiles_pay(const GemmParams &p, double penalty) {
+  if (p.block_tile != 0) return p.block_tile == 2;
+  const size_t units = (size_t)compute_units();
+  auto busy = [&](size_t bx, size_t by) {
+    const size_t tiles = (size_t)p.batch * ceil_div((size_t)p.nx, bx) * ceil_div((size_t)p.ny, by);
+    return (double)tiles / (double)(units * ceil_div(tiles, units));
+  };
+  return busy(128, 128) / penalty > busy(256, 128);
+}
+
 template <int DT, int TOUT>
 hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   constexpr int KPM = DtypeTraits<DT>::kTilesPerMfma;
@@ -1985,12 +2001,25 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
           return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, false>(p, stream);
         }
       }
+      // problems too small to give every compute unit a 256 x 128 tile: 128 x 128
+      // blocks, 8 waves of 64 x 32, 4-slot ring
+      if (small_tiles_pay(p, 1.15)) {
+        return p.variant == kOpt
+                   ? launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>(p, stream)
+                   : launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadPlanarVec, 16>(p, stream);
+      }
       return p.variant == kOpt
                  ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>(p, stream)
                  : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>(p, stream);
     } else {
       // fp8: the 32x32x64 MFMA takes one K tile per instruction, which lets the
       // same block shape and ring as for 16-bit input fit into LDS
+      // (small problems: 128 x 128 blocks, 4 waves of 64 x 64, two blocks a unit)
+      if (small_tiles_pay(p, 1.05)) {
+        return p.variant == kOpt
+                   ? launch_dtl<DT, TOUT, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>(p, stream)
+                   : launch_dtl<DT, TOUT, 128, 128, 64, 64, 2, 2, kLoadPlanarVec, 32>(p, stream);
+      }
       return p.variant == kOpt
                  ? launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
                  : launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
@@ -2029,6 +2058,11 @@ hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
       // packed 1-bit samples expanded in registers; the caller has checked that
       // planar rows are whole aligned 16-byte chunks and that K fits fp32 sums
       if (p.type_out == kInt32 && !p.input_interleaved) {
+        if (small_tiles_pay(p, 1.0)) {
+          return p.variant == kOpt
+                     ? launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>(p, stream)
+                     : launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadPlanarVec, 32>(p, stream);
+        }
         return p.variant == kOpt
                    ? launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
                    : launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);

@@ -47,6 +47,9 @@ static const std::vector<Config> kConfigs = {
     {"bf16 256x128 w64x64 s3 m16", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kBfloat16, kFloat32},
     {"f32 256x128 w64x64 s3 m16", launch_dtl<kFloat32, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat32, kFloat32},
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
+    {"fp8 128x128 w64x64 s2 m32", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
+    {"fp8 128x128 w64x32 s4 m32", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
+    {"int1 128x128 w64x64 s2 m32", launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>, kInt1, kInt32},
     {"int1 256x128 w64x64 s3 m32", launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kInt1, kInt32},
     // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},

@@ -84,12 +84,17 @@ CCGLIB_API const char *ccglib_version(void);
  *                    or more in chunks of whole batches of about 32 MiB; any
  *                    other value: chunks of about that many bytes, whatever
  *                    the size of the job.
+ *   GEMM_BLOCK_TILE  0 (default): GEMMs on tiled or whole-chunk planar
+ *                    operands use 256 x 128 block tiles, or 128 x 128 ones
+ *                    when the larger would leave compute units idle (small
+ *                    problems); 1: always 256 x 128; 2: always 128 x 128.
  * ---------------------------------------------------------------------- */
 enum {
   CCGLIB_AMD_OPTION_INT1_POPCOUNT = 0,
   CCGLIB_AMD_OPTION_BASIC_RETILE = 1,
   CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES = 2,
-  CCGLIB_AMD_OPTION_COUNT = 3
+  CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE = 3,
+  CCGLIB_AMD_OPTION_COUNT = 4
 };
 CCGLIB_API int ccglib_amd_set_option(int option, size_t value);
 CCGLIB_API int ccglib_amd_get_option(int option, size_t *value);

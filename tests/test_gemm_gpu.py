@@ -423,3 +423,47 @@ def test_int1_k_in_pieces(variant, K, int1_kernel):
 def test_int1_alpha_beta(variant, int1_kernel):
     # test/gemm/mma.cpp:713-775
     int1_case(16, 256, 128, 256, variant, alpha=2 - 3j, beta=3 - 2j)
+
+
+# ---- both block tiles of the MFMA kernels ------------------------------------------------
+
+@pytest.mark.parametrize("block_tile", [1, 2])
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.bfloat16, VT.bfloat16),
+                                      (VT.float32, VT.float16), (VT.float8e4m3, VT.float32)])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_block_tiles(block_tile, tin, tout, variant):
+    """The dispatch picks 256 x 128 or 128 x 128 block tiles by problem size (option
+    GEMM_BLOCK_TILE = 0); here each is forced in turn on the same problems: one
+    partial tile, many tiles with ragged edges, a long K, alpha / beta, column-major
+    and (opt) interleaved C."""
+    with cc.option(cc.Option.gemm_block_tile, block_tile):
+        float_case(1, 70, 50, 40, tin, tout, variant, PLANAR, ROW, seed=1)
+        float_case(2, 300, 520, 96, tin, tout, variant, PLANAR, COL, seed=2)
+        float_case(1, 130, 260, 1064, tin, tout, variant, PLANAR, ROW, alpha=1.5 - 0.5j, beta=0.25 + 1j,
+                   seed=3)
+        if variant == cc.Variant.opt:
+            float_case(3, 257, 129, 72, tin, tout, variant, INTERLEAVED, ROW, alpha=2j, seed=4)
+
+
+@pytest.mark.parametrize("block_tile", [1, 2])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+def test_block_tiles_int1(block_tile, variant):
+    with cc.option(cc.Option.gemm_block_tile, block_tile):
+        int1_case(2, 70, 50, 640, variant, seed=1)
+        int1_case(3, 300, 520, 1536, variant, c_order=COL, alpha=2 - 1j, beta=1 + 3j, seed=2)
+        int1_case(1, 257, 129, 4096 + 512, variant, seed=3)
+        if variant == cc.Variant.opt:
+            int1_case(2, 130, 260, 1024, variant, c_axis=INTERLEAVED, seed=4)
+
+
+def test_block_tile_choice_is_invisible():
+    """The same bits whichever block tile computes them (same K order per element)."""
+    rng = np.random.default_rng(11)
+    B, M, N, K = 2, 384, 640, 256
+    qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), VT.float16).reshape(-1)
+    qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), VT.float16).reshape(-1)
+    results = []
+    for block_tile in (0, 1, 2):
+        with cc.option(cc.Option.gemm_block_tile, block_tile):
+            results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt))
+    assert np.array_equal(results[0], results[1]) and np.array_equal(results[1], results[2])
