@@ -1984,8 +1984,14 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     if constexpr (DT == kFloat32) {
       return hipErrorInvalidValue;
     } else if constexpr (KPM == 1) {
+      if (small_tiles_pay(p, 1.15)) {
+        return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec>(p, stream);
+      }
       return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec>(p, stream);
     } else {
+      if (small_tiles_pay(p, 1.05)) {
+        return launch_dtl<DT, TOUT, 128, 128, 64, 64, 2, 2, kLoadInterleavedVec, 32>(p, stream);
+      }
       return launch_dtl<DT, TOUT, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>(p, stream);
     }
   }

@@ -343,3 +343,30 @@ def test_pipeline_basic_rejects_interleaved_output():
     with pytest.raises(RuntimeError, match="complex-interleaved output is not supported in basic variant"):
         cc.Pipeline(1, 16, 16, 16, 0, stream(), PLANAR, INTERLEAVED, ROW, COL, ROW, VT.float16,
                     VT.float32, cc.Variant.basic)
+
+
+@pytest.mark.parametrize("block_tile", [1, 2])
+@pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
+def test_pipeline_interleaved_rows_read_in_place_with_either_block_tile(block_tile, tin):
+    """8- and 16-bit interleaved input whose rows are whole 16-byte chunks is read by the
+    GEMM in place; its kernel has the same two block tiles as the tiled one (option
+    GEMM_BLOCK_TILE forces one)."""
+    B, M, N, K = 3, 300, 260, 160
+    rng = np.random.default_rng(7)
+    qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), tin)
+    qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), tin)
+    qa_il = np.ascontiguousarray(qa.transpose(0, 2, 3, 1)).reshape(-1)
+    qb_il = np.ascontiguousarray(qb.transpose(0, 2, 3, 1)).reshape(-1)
+    with cc.option(cc.Option.gemm_block_tile, block_tile):
+        p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, tin, VT.float32,
+                        cc.Variant.opt, 0.5 + 1j)
+    d_a, d_b = to_device(qa_il), to_device(qb_il)
+    d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
+    p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, np.float32).reshape(B, 2, M, N)
+    want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], orc.FLOAT32, orc.ROW_MAJOR,
+                    0.5 + 1j)
+    w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin])
+    w = (w64[:, 0] + 1j * w64[:, 1]) * (0.5 + 1j)
+    check_float(got, want, np.stack([w.real, w.imag], 1), tin, VT.float32)
