@@ -774,13 +774,22 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
   const bool fused = allow_fused && !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&
                      (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2800.0 : 3000.0));
+  // Planar input of the opt variant whose rows are whole 16-byte chunks: the GEMM
+  // can read the rows in place as well (the basic variant's loader, same
+  // arithmetic and K order as on tiles). That costs the GEMM 9-12 %, so the
+  // break-even against the two transposes lies lower, at about 1750.
+  const bool planar_in_place = allow_fused && !packing && variant == kOpt &&
+                               input_complex_axis_location == kPlanar &&
+                               output_complex_axis_location == kPlanar && K > 0 &&
+                               (in_bits == 8 || in_bits == 16 || in_bits == 32) &&
+                               (K * in_bits / 8) % 16 == 0 && mn_over_sum < 1750.0;
   // The reference transposes for the opt variant only (:53) and hands interleaved
   // input of the basic variant to a kernel that reads it as planar. Here such
   // input is always de-interleaved: in the GEMM's loader (fused) or, where that
   // cannot take the rows, by the transposes, with the tiled kernel behind them.
   const bool basic_needs_tiles = !packing && variant == kBasic &&
                                  input_complex_axis_location == kInterleaved && !fused;
-  const bool transposing = ((variant == kOpt) && !fused) || basic_needs_tiles;
+  const bool transposing = ((variant == kOpt) && !fused && !planar_in_place) || basic_needs_tiles;
   // Packing moves the real samples of every batch in front of its imaginary ones
   // (below), so what follows it sees planar data. (The reference hands
   // input_complex_axis_location to its Transpose here too,
@@ -870,12 +879,14 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
       }
     }
     rc = ccglib_gemm_create(&p->gemm, B, M, N, K, device, stream, input_type, output_type,
-                            (fused || basic_needs_tiles) ? (int)kOpt : variant,
+                            (fused || basic_needs_tiles) ? (int)kOpt
+                            : planar_in_place            ? (int)kBasic
+                                                         : variant,
                             output_complex_axis_location,
                             c_mem_order, a_mem_order, b_mem_order, alpha_re, alpha_im, beta_re,
                             beta_im);  // :102-105
     if (rc == CCGLIB_OK) p->gemm->input_interleaved = fused;
-    p->fused = fused;
+    p->fused = fused || planar_in_place;   // (both need 16-byte aligned rows at Run)
   } while (false);
   if (rc != CCGLIB_OK) {
     const std::string keep = g_last_error;

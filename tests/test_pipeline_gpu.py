@@ -370,3 +370,36 @@ def test_pipeline_interleaved_rows_read_in_place_with_either_block_tile(block_ti
     w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin])
     w = (w64[:, 0] + 1j * w64[:, 1]) * (0.5 + 1j)
     check_float(got, want, np.stack([w.real, w.imag], 1), tin, VT.float32)
+
+
+@pytest.mark.parametrize("tin,K", [(VT.float16, 96), (VT.float8e5m2, 144), (VT.float32, 36)])
+@pytest.mark.parametrize("skew", [0, 1])
+def test_pipeline_planar_rows_read_in_place(tin, K, skew):
+    """Planar input of the opt variant whose rows are whole 16-byte chunks is read by the
+    GEMM in place when the two transposes would cost more than they save (small
+    M N / (M + N)); the result has the bits of Transpose + opt GEMM on the same data.
+    skew: buffers one element off a 16-byte boundary, for which the pipeline falls
+    back to its transposes."""
+    from gpu_util import transpose_operand
+    B, M, N = 3, 200, 300
+    tout = VT.float32
+    rng = np.random.default_rng(K)
+    qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), tin).reshape(-1)
+    qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), tin).reshape(-1)
+    pad = np.zeros(skew, dtype=qa.dtype)
+    d_a, d_b = to_device(np.concatenate([pad, qa])), to_device(np.concatenate([pad, qb]))
+    off = skew * qa.dtype.itemsize
+    d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
+    p = cc.Pipeline(B, M, N, K, 0, stream(), PLANAR, PLANAR, ROW, COL, ROW, tin, tout, cc.Variant.opt)
+    p.Run(d_a.data_ptr() + off, d_b.data_ptr() + off, d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, np.float32).reshape(B, 2, M, N)
+    want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[tin], orc.FLOAT32)
+    check_float(got, want, orc.gemm_float64(qa, qb, M, N, K, ORC_TYPE[tin]), tin, tout)
+    # the reference's sequence with separate objects
+    t_a, t_b = transpose_operand(qa, B, M, K, tin), transpose_operand(qb, B, N, K, tin)
+    d_c2 = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
+    cc.GEMM(B, M, N, K, 0, stream(), cc.Precision(tin, tout), cc.Variant.opt).Run(
+        t_a.data_ptr(), t_b.data_ptr(), d_c2.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(got.reshape(-1), to_host(d_c2, np.float32))
