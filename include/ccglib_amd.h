@@ -213,7 +213,9 @@ CCGLIB_API int ccglib_packing_destroy(ccglib_packing_t packing);
  * as one, kernels/packing_kernel.cu:15-22, which is the same for B = 1); the
  * opt variant transposes A and B first. 8- and 16-bit interleaved input whose
  * rows are whole 16-byte chunks is read by the GEMM in place instead (no
- * transposes); if a Run then gets pointers that are not 16-byte aligned, the
+ * transposes), and so is planar input of the opt variant with such rows when
+ * the problem is small enough for the transposes to cost more than they save;
+ * if a Run then gets pointers that are not 16-byte aligned, the
  * object builds the pipeline with transposes at that Run and uses it for such
  * calls. Argument order follows the reference constructor.
  * run_host copies a, b (and c when beta != 0) to the device, runs, copies c
