@@ -1391,16 +1391,17 @@ __global__ __launch_bounds__(64 * (BX / WX) * (BY / WY), WAVES_PER_EU) void comp
 // fetch the chunk that belongs there (a permutation inside each 64-byte row,
 // so the global access stays fully coalesced).
 //
-// LDS is a ring of SLOTS K tiles. Iteration i waits for its own tile(s) with
-// s_waitcnt vmcnt(n) - n being the loads issued for later iterations - then
-// passes one barrier, issues the loads LEAD iterations ahead into the slot(s)
-// that the previous iteration just released, and does the math.
+// LDS is a ring of SLOTS K tiles (X and Y may have rings of different depth).
+// Iteration i waits for its own tile with s_waitcnt vmcnt(n) - n being the
+// loads issued for later iterations - then passes one barrier, issues the loads
+// SLOTS - 1 iterations ahead into the slot that the previous iteration just
+// released (after its first group of MFMAs), and does the math.
 //
 // Blocks are persistent: each walks a sequence of C tiles, and the copy simply
 // runs on into the next C tile, so its first K tiles are in flight while the
 // current tile's results are stored, and those stores drain under the next
-// tile's math. Loads past the end of K (an odd fp8 tile count) or past the
-// last C tile are pointed at a zero tile, which keeps the number of
+// tile's math. Loads past the end of K (rows whose last K tile is partial) or
+// past the last C tile are pointed at a zero tile, which keeps the number of
 // outstanding loads the same in every iteration.
 // ---------------------------------------------------------------------------
 __device__ __attribute__((aligned(256))) char g_zero_tile[kTileBytes];
