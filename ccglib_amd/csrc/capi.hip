@@ -796,7 +796,7 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
   // src/pipeline/Pipeline.cpp:78-84, which then de-interleaves packed words.)
   const int axis_after_packing = packing ? kPlanar : input_complex_axis_location;
   do {
-    if (packing && input_complex_axis_location == kPlanar && B && M && N && K % 32 == 0) {
+    if (packing && B && M && N && K % 32 == 0) {
       // (K in whole words, as the packed layout of the other route needs it.)
       // The 1-bit GEMM multiplies operands expanded to 4-bit values; when its
       // workspace holds the whole problem the expansion is done straight from
@@ -823,6 +823,8 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
       fill_gemm_params(p->gemm, nullptr, nullptr, nullptr, &probe);
       if (gemm_int1_can_take_bytes(probe)) {
         p->int1_direct = true;
+        // (interleaved bytes are de-interleaved while they are packed into tiles)
+        p->gemm->input_interleaved = (input_complex_axis_location == kInterleaved);
         break;
       }
       ccglib_gemm_destroy(p->gemm);
@@ -1182,6 +1184,27 @@ int ccglib_pipeline_run_static(size_t B, size_t M, size_t N, size_t K, int devic
   size_t tiled_a = 0, tiled_b = 0;
   tiled_bytes(&g, &tiled_a, &tiled_b);
   const bool pack_first = int1 && input_complex_axis_location == kInterleaved;
+  if (int1 && tiled_a + tiled_b <= kStaticScratchBytes) {
+    // one byte per sample, planar or (re, im) pairs: packed straight into 1-bit
+    // tiles (A's and B's back to back), then multiplied
+    g.workspace = ws;
+    g.workspace_bytes = tiled_a + tiled_b;
+    g.input_interleaved = pack_first;
+    GemmParams q;
+    fill_gemm_params(&g, d_a, d_b, d_c, &q);
+    q.int1_direct = 1;
+    if (gemm_int1_can_take_bytes(q)) {
+      const hipError_t e = launch_gemm_int1_from_bytes(q, s);
+      if (e != hipSuccess) return fail_hip(e, "1-bit pipeline launch");
+      return CCGLIB_OK;
+    }
+    if (!pack_first) {
+      return fail(CCGLIB_ERROR_UNSUPPORTED, "ccglib_pipeline_run_static: 1-bit problem out of range");
+    }
+    g.workspace = nullptr;
+    g.workspace_bytes = 0;
+    g.input_interleaved = false;
+  }
   const size_t packed_a = pack_first ? round_up_256(B * 2 * M * K / 8) : 0;
   const size_t packed_b = pack_first ? round_up_256(B * 2 * N * K / 8) : 0;
   const size_t need = round_up_256(tiled_a) + round_up_256(tiled_b) + packed_a + packed_b;
@@ -1193,22 +1216,6 @@ int ccglib_pipeline_run_static(size_t B, size_t M, size_t N, size_t K, int devic
   }
   unsigned char *ws_a = ws, *ws_b = ws + round_up_256(tiled_a);
   unsigned char *ws_pa = ws_b + round_up_256(tiled_b), *ws_pb = ws_pa + packed_a;
-
-  if (int1 && !pack_first) {
-    // one byte per sample, planar: packed straight into 1-bit tiles, then multiplied
-    g.workspace = ws;
-    g.workspace_bytes = tiled_a + tiled_b;
-    GemmParams q;
-    fill_gemm_params(&g, d_a, d_b, d_c, &q);
-    q.int1_direct = 1;
-    if (!gemm_int1_can_take_bytes(q)) {
-      return fail(CCGLIB_ERROR_UNSUPPORTED, "ccglib_pipeline_run_static: 1-bit problem out of range");
-    }
-    // (the packing kernel writes A's tiles and B's tiles back to back)
-    const hipError_t e = launch_gemm_int1_from_bytes(q, s);
-    if (e != hipSuccess) return fail_hip(e, "1-bit pipeline launch");
-    return CCGLIB_OK;
-  }
 
   const void *src_a = d_a, *src_b = d_b;
   int axis = input_complex_axis_location;

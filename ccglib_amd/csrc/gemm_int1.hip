@@ -317,6 +317,90 @@ hipError_t launch_int1_on_mfma(const GemmParams &p, hipStream_t stream, bool *do
   return hipSuccess;   // not done: the caller runs the vector-ALU kernel
 }
 
+// The same for interleaved input ([batch][rows][K][2] bytes, (re, im) pairs): a
+// wave takes eight rows of one K tile, a whole row of 512 samples (1 KiB) per
+// load instruction, eight loads in flight. A lane's 16 bytes are eight pairs:
+// eight real and eight imaginary bits, a quarter word of each plane; the four
+// lanes of a quad exchange theirs (three DPP moves) and the first two of them
+// store the real and the imaginary word, so a store instruction of a wave
+// writes one 64-byte tile row in each plane. Samples keep their order here
+// (sample k of a row's tile is bit k % 32 of word k / 32): both operands of a
+// pipeline have the same layout and are packed by the same kernel.
+__device__ __forceinline__ unsigned nonzero_nibble(unsigned x) {
+  const unsigned nz = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
+  return (((nz >> 7) * 0x00204081u) >> 21) & 0xfu;
+}
+
+// 8 (re, im) byte pairs -> real bits in bits 0-7, imaginary bits in bits 8-15
+__device__ __forceinline__ unsigned pair_bits(uint4_t v) {
+  const unsigned re_lo = __builtin_amdgcn_perm(v[1], v[0], 0x06040200u);
+  const unsigned re_hi = __builtin_amdgcn_perm(v[3], v[2], 0x06040200u);
+  const unsigned im_lo = __builtin_amdgcn_perm(v[1], v[0], 0x07050301u);
+  const unsigned im_hi = __builtin_amdgcn_perm(v[3], v[2], 0x07050301u);
+  return nonzero_nibble(re_lo) | (nonzero_nibble(re_hi) << 4) | (nonzero_nibble(im_lo) << 8) |
+         (nonzero_nibble(im_hi) << 12);
+}
+
+constexpr unsigned kPairRowsPerWave = 8;
+template <bool VEC>
+__global__ __launch_bounds__(256) void pack_pairs_to_tiles(const unsigned char *__restrict__ src,
+                                                           char *__restrict__ dst, unsigned rows,
+                                                           unsigned row_tiles, unsigned k,
+                                                           unsigned k1_tiles) {
+  // blockIdx: x = four K tiles of 512 samples (one per wave: a block reads 4 KiB
+  // contiguous of each of its rows), y = block of eight rows, z = batch
+  const unsigned lane = threadIdx.x & 63;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr unsigned RPW = kPairRowsPerWave, WPT = kTileRows / RPW;
+  const unsigned rt = blockIdx.y / WPT;
+  const unsigned row0_in_tile = (blockIdx.y % WPT) * RPW;
+  const size_t b = blockIdx.z;
+  const unsigned kt = blockIdx.x * 4 + wave;
+  if (kt >= k1_tiles) return;
+  const unsigned k0 = kt * 512 + lane * 8;      // first of this lane's eight samples
+  unsigned bits[RPW];
+  // the same for all threads of a wave: all its rows and all 512 samples exist
+  if (VEC && rt * kTileRows + row0_in_tile + RPW <= rows && kt * 512 + 512 <= k) {
+    const unsigned char *p0 = src + ((b * rows + rt * kTileRows + row0_in_tile) * (size_t)k + k0) * 2;
+    uint4_t v[RPW];
+#pragma unroll
+    for (unsigned i = 0; i < RPW; ++i) {
+      v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(p0 + (size_t)i * k * 2));
+    }
+#pragma unroll
+    for (unsigned i = 0; i < RPW; ++i) bits[i] = pair_bits(v[i]);
+  } else {
+#pragma unroll
+    for (unsigned i = 0; i < RPW; ++i) {
+      const unsigned r = rt * kTileRows + row0_in_tile + i;
+      const unsigned char *row_ptr = src + (b * rows + (r < rows ? r : 0)) * (size_t)k * 2;
+      const unsigned n = (r < rows && k0 < k) ? (k - k0 < 8 ? k - k0 : 8) : 0;
+      unsigned re = 0, im = 0;
+      for (unsigned e = 0; e < n; ++e) {
+        re |= (row_ptr[2 * (size_t)(k0 + e)] != 0 ? 1u : 0u) << e;
+        im |= (row_ptr[2 * (size_t)(k0 + e) + 1] != 0 ? 1u : 0u) << e;
+      }
+      bits[i] = re | (im << 8);
+    }
+  }
+  // lanes 4 w .. 4 w + 3 hold the four bytes of word w of either plane
+  const unsigned plane = lane & 1;
+  char *out = dst + ((b * row_tiles + rt) * k1_tiles + kt) * kTileBytes + plane * kTilePlaneBytes +
+              row0_in_tile * kTileRowBytes + 4 * (lane >> 2);
+#pragma unroll
+  for (unsigned i = 0; i < RPW; ++i) {
+    const int mine = (int)bits[i];
+    const unsigned q0 = (unsigned)__builtin_amdgcn_update_dpp(0, mine, 0x00, 0xf, 0xf, false);
+    const unsigned q1 = (unsigned)__builtin_amdgcn_update_dpp(0, mine, 0x55, 0xf, 0xf, false);
+    const unsigned q2 = (unsigned)__builtin_amdgcn_update_dpp(0, mine, 0xAA, 0xf, 0xf, false);
+    const unsigned q3 = (unsigned)__builtin_amdgcn_update_dpp(0, mine, 0xFF, 0xf, 0xf, false);
+    const unsigned sh = plane * 8;
+    const unsigned word = ((q0 >> sh) & 0xffu) | (((q1 >> sh) & 0xffu) << 8) |
+                          (((q2 >> sh) & 0xffu) << 16) | (((q3 >> sh) & 0xffu) << 24);
+    if ((lane & 3) < 2) *reinterpret_cast<unsigned *>(out + i * kTileRowBytes) = word;
+  }
+}
+
 }  // namespace
 
 bool gemm_int1_can_take_bytes(const GemmParams &p) {
@@ -334,6 +418,19 @@ hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) 
   for (int which = 0; which < 2; ++which) {
     const unsigned rows = which ? p.ny : p.nx, row_tiles = which ? p.y_tiles : p.x_tiles;
     const unsigned char *src = static_cast<const unsigned char *>(which ? p.y : p.x);
+    if (p.input_interleaved) {
+      // (re, im) byte pairs
+      const dim3 grid((unsigned)ceil_div(k1_tiles, 4), (kTileRows / kPairRowsPerWave) * row_tiles, p.batch);
+      const bool vec = (p.k % 8 == 0) && ((uintptr_t)src % 16 == 0);
+      if (vec) {
+        hipLaunchKernelGGL(pack_pairs_to_tiles<true>, grid, dim3(256), 0, stream, src,
+                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
+      } else {
+        hipLaunchKernelGGL(pack_pairs_to_tiles<false>, grid, dim3(256), 0, stream, src,
+                           which ? ws_y : ws_x, rows, row_tiles, p.k, k1_tiles);
+      }
+      continue;
+    }
     const dim3 grid((unsigned)ceil_div(k1_tiles, 4), (kTileRows / (2 * kPackLoads)) * row_tiles, 2 * p.batch);
     const bool vec = (p.k % 16 == 0) && ((uintptr_t)src % 16 == 0);
     if (vec) {
@@ -349,6 +446,7 @@ hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream) 
   q.x = ws_x;
   q.y = ws_y;
   q.variant = kOpt;
+  q.input_interleaved = 0;   // (the tiles are planar whatever the bytes were)
   q.k_tiles = k1_tiles;
   return launch_gemm_mfma(q, stream);
 }
