@@ -208,9 +208,12 @@ CCGLIB_API int ccglib_packing_destroy(ccglib_packing_t packing);
  * Run(device) :54 (src/pipeline/Pipeline.cpp:183-188), Run(host) :41
  * (src/pipeline/Pipeline.cpp:162-176).
  * 1-bit input is one byte per sample and is packed first (interleaved input:
- * every batch on its own, real bits then imaginary bits, which needs M*K and
- * N*K to be multiples of 32 when B > 1; the reference packs the whole buffer
- * as one, kernels/packing_kernel.cu:15-22, which is the same for B = 1); the
+ * every batch on its own, real bits then imaginary bits; the reference packs
+ * the whole buffer as one, kernels/packing_kernel.cu:15-22, which is the same
+ * for B = 1. With K a multiple of 32 the bytes go straight into the GEMM's
+ * 1-bit tiles; otherwise, and with CCGLIB_AMD_OPTION_INT1_POPCOUNT, through a
+ * packed buffer, which for interleaved input and B > 1 needs M*K and N*K to be
+ * multiples of 32); the
  * opt variant transposes A and B first. 8- and 16-bit interleaved input whose
  * rows are whole 16-byte chunks is read by the GEMM in place instead (no
  * transposes), and so is planar input of the opt variant with such rows when
