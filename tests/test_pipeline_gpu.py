@@ -403,3 +403,8 @@ def test_pipeline_planar_rows_read_in_place(tin, K, skew):
         t_a.data_ptr(), t_b.data_ptr(), d_c2.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(got.reshape(-1), to_host(d_c2, np.float32))
+    # and the host Run of the same object
+    if skew == 0:
+        host_c = np.full(B * 2 * M * N, np.nan, dtype=np.float32)
+        p.RunHost(qa.ctypes.data, qb.ctypes.data, host_c.ctypes.data)
+        assert np.array_equal(host_c, got.reshape(-1))
