@@ -13,8 +13,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libccglib_amd.so")
-SOURCES = ["capi.hip", "gemm_mfma.hip", "gemm_int1.hip", "transpose.hip", "packing.hip"]
+# (gemm_mfma.hip is compiled in parts, one per input type, so that they build in parallel)
+SOURCES = ["capi.hip", "gemm_mfma_f16.hip", "gemm_mfma_bf16.hip", "gemm_mfma_f32.hip",
+           "gemm_mfma_fp8.hip", "gemm_mfma_int1.hip", "gemm_mfma_dispatch.hip", "gemm_int1.hip",
+           "transpose.hip", "packing.hip"]
 HEADERS = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_device.h"),
+           os.path.join(CSRC, "gemm_mfma.hip"),
            os.path.join(os.path.dirname(HERE), "include", "ccglib_amd.h")]
 
 # Packed-fp32 instruction selection is switched off for all device code.

@@ -2040,45 +2040,83 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
 
 }  // namespace
 
-hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
-  switch (p.type_in) {
-    case kFloat16:
-      if (p.type_out == kFloat32) return launch_typed<kFloat16, kFloat32>(p, stream);
-      if (p.type_out == kFloat16) return launch_typed<kFloat16, kFloat16>(p, stream);
-      break;
-    case kBfloat16:
-      if (p.type_out == kFloat32) return launch_typed<kBfloat16, kFloat32>(p, stream);
-      if (p.type_out == kBfloat16) return launch_typed<kBfloat16, kBfloat16>(p, stream);
-      break;
-    case kFloat32:
-      if (p.type_out == kFloat32) return launch_typed<kFloat32, kFloat32>(p, stream);
-      if (p.type_out == kFloat16) return launch_typed<kFloat32, kFloat16>(p, stream);
-      if (p.type_out == kBfloat16) return launch_typed<kFloat32, kBfloat16>(p, stream);
-      break;
-    case kFloat8e4m3:
-      if (p.type_out == kFloat32) return launch_typed<kFloat8e4m3, kFloat32>(p, stream);
-      break;
-    case kFloat8e5m2:
-      if (p.type_out == kFloat32) return launch_typed<kFloat8e5m2, kFloat32>(p, stream);
-      break;
-    case kInt1:
-      // packed 1-bit samples expanded in registers; the caller has checked that
-      // planar rows are whole aligned 16-byte chunks and that K fits fp32 sums
-      if (p.type_out == kInt32 && !p.input_interleaved) {
-        if (small_tiles_pay(p, 1.0)) {
-          return p.variant == kOpt
-                     ? launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>(p, stream)
-                     : launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadPlanarVec, 32>(p, stream);
-        }
-        return p.variant == kOpt
-                   ? launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
-                   : launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
-      }
-      break;
-    default:
-      break;
-  }
+// The instantiations are spread over several translation units so that they
+// compile in parallel: gemm_mfma_<part>.hip define CCGLIB_GEMM_MFMA_PART and
+// include this file (1 fp16, 2 bf16, 3 fp32, 4 fp8, 5 1-bit input; 0 the
+// dispatch below). Included without the macro (the tuning program), the file
+// holds everything.
+#ifndef CCGLIB_GEMM_MFMA_PART
+#define CCGLIB_GEMM_MFMA_PART -1
+#endif
+#define CCGLIB_GEMM_MFMA_HAS(part) (CCGLIB_GEMM_MFMA_PART == -1 || CCGLIB_GEMM_MFMA_PART == (part))
+
+hipError_t launch_gemm_mfma_f16(const GemmParams &p, hipStream_t stream);
+hipError_t launch_gemm_mfma_bf16(const GemmParams &p, hipStream_t stream);
+hipError_t launch_gemm_mfma_f32(const GemmParams &p, hipStream_t stream);
+hipError_t launch_gemm_mfma_fp8(const GemmParams &p, hipStream_t stream);
+hipError_t launch_gemm_mfma_int1(const GemmParams &p, hipStream_t stream);
+
+#if CCGLIB_GEMM_MFMA_HAS(1)
+hipError_t launch_gemm_mfma_f16(const GemmParams &p, hipStream_t stream) {
+  if (p.type_out == kFloat32) return launch_typed<kFloat16, kFloat32>(p, stream);
+  if (p.type_out == kFloat16) return launch_typed<kFloat16, kFloat16>(p, stream);
   return hipErrorInvalidValue;
 }
+#endif
+
+#if CCGLIB_GEMM_MFMA_HAS(2)
+hipError_t launch_gemm_mfma_bf16(const GemmParams &p, hipStream_t stream) {
+  if (p.type_out == kFloat32) return launch_typed<kBfloat16, kFloat32>(p, stream);
+  if (p.type_out == kBfloat16) return launch_typed<kBfloat16, kBfloat16>(p, stream);
+  return hipErrorInvalidValue;
+}
+#endif
+
+#if CCGLIB_GEMM_MFMA_HAS(3)
+hipError_t launch_gemm_mfma_f32(const GemmParams &p, hipStream_t stream) {
+  if (p.type_out == kFloat32) return launch_typed<kFloat32, kFloat32>(p, stream);
+  if (p.type_out == kFloat16) return launch_typed<kFloat32, kFloat16>(p, stream);
+  if (p.type_out == kBfloat16) return launch_typed<kFloat32, kBfloat16>(p, stream);
+  return hipErrorInvalidValue;
+}
+#endif
+
+#if CCGLIB_GEMM_MFMA_HAS(4)
+hipError_t launch_gemm_mfma_fp8(const GemmParams &p, hipStream_t stream) {
+  if (p.type_out != kFloat32) return hipErrorInvalidValue;
+  return p.type_in == kFloat8e4m3 ? launch_typed<kFloat8e4m3, kFloat32>(p, stream)
+                                  : launch_typed<kFloat8e5m2, kFloat32>(p, stream);
+}
+#endif
+
+#if CCGLIB_GEMM_MFMA_HAS(5)
+hipError_t launch_gemm_mfma_int1(const GemmParams &p, hipStream_t stream) {
+  // packed 1-bit samples expanded in registers; the caller has checked that
+  // planar rows are whole aligned 16-byte chunks and that K fits fp32 sums
+  if (p.type_out != kInt32 || p.input_interleaved) return hipErrorInvalidValue;
+  if (small_tiles_pay(p, 1.0)) {
+    return p.variant == kOpt
+               ? launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>(p, stream)
+               : launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadPlanarVec, 32>(p, stream);
+  }
+  return p.variant == kOpt
+             ? launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>(p, stream)
+             : launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>(p, stream);
+}
+#endif
+
+#if CCGLIB_GEMM_MFMA_HAS(0)
+hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
+  switch (p.type_in) {
+    case kFloat16: return launch_gemm_mfma_f16(p, stream);
+    case kBfloat16: return launch_gemm_mfma_bf16(p, stream);
+    case kFloat32: return launch_gemm_mfma_f32(p, stream);
+    case kFloat8e4m3:
+    case kFloat8e5m2: return launch_gemm_mfma_fp8(p, stream);
+    case kInt1: return launch_gemm_mfma_int1(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+#endif
 
 }  // namespace ccglib_amd
