@@ -18,7 +18,7 @@ SOURCES = ["capi.hip", "gemm_mfma_f16.hip", "gemm_mfma_bf16.hip", "gemm_mfma_f32
            "gemm_mfma_fp8.hip", "gemm_mfma_int1.hip", "gemm_mfma_dispatch.hip", "gemm_int1.hip",
            "transpose.hip", "packing.hip"]
 HEADERS = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_device.h"),
-           os.path.join(CSRC, "gemm_mfma.hip"),
+           os.path.join(CSRC, "gemm_mfma.hip"), os.path.join(CSRC, "gemm_mfma_wide.h"),
            os.path.join(os.path.dirname(HERE), "include", "ccglib_amd.h")]
 
 # Packed-fp32 instruction selection is switched off for all device code.

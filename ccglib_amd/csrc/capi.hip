@@ -327,8 +327,8 @@ int ccglib_amd_set_option(int option, size_t value) {
   if (option < 0 || option >= CCGLIB_AMD_OPTION_COUNT) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "unknown option %d", option);
   }
-  if (option == CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE && value > 2) {
-    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "GEMM_BLOCK_TILE is 0, 1 or 2 (got %zu)", value);
+  if (option == CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE && value > 3) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "GEMM_BLOCK_TILE is 0, 1, 2 or 3 (got %zu)", value);
   }
   g_options[option] = value;
   return CCGLIB_OK;

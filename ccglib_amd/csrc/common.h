@@ -84,7 +84,7 @@ struct GemmParams {
   // 1-bit GEMM only: the MFMA kernel may multiply the packed words (0: the
   // vector-ALU kernel runs whatever the layout)
   int int1_direct = 1;
-  int block_tile = 0;      // 0: chosen per problem; 1: 256 x 128 blocks; 2: 128 x 128 blocks
+  int block_tile = 0;      // 0: chosen per problem; 1: 256 x 128 blocks; 2: 128 x 128; 3: 192 x 256
 };
 
 // Bytes of both operands in the tiled 1-bit layout (what the pipeline packs the

@@ -28,11 +28,24 @@
 //  * Workgroup ids are remapped so that consecutive tiles land on the same
 //    XCD (shared L2), in groups that reuse both operands.
 #include <atomic>
+#include <type_traits>
 
 #include "gemm_device.h"
 
+// Timing-only builds for the kernel-configuration sweep (never for the library):
+// a bit mask of parts of the kernels to leave out, which gives wrong numbers and
+// shows what each part costs. 1: the C stores (of the register-direct epilogues of
+// 16-bit input); 2: the matrix instructions (16-row shapes); 4: the global -> LDS
+// copies; 8: the barrier of the K loop.
+#ifndef CCGLIB_ABLATE
+#define CCGLIB_ABLATE 0
+#endif
+
 namespace ccglib_amd {
 namespace {
+
+constexpr bool kAblateStores = (CCGLIB_ABLATE & 1) != 0, kAblateMfma = (CCGLIB_ABLATE & 2) != 0,
+               kAblateCopies = (CCGLIB_ABLATE & 4) != 0, kAblateBarrier = (CCGLIB_ABLATE & 8) != 0;
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -60,6 +73,11 @@ template <int DT> struct Fragment {
 template <int DT>
 __device__ __forceinline__ float4_t mfma(const Fragment<DT> &a, const Fragment<DT> &b,
                                          float4_t acc) {
+  if constexpr (kAblateMfma) {
+    // (timing-only build: the operands are still fetched)
+    asm volatile("" : "+v"(acc) : "v"(a.v[0]), "v"(b.v[0]));
+    return acc;
+  }
   if constexpr (DT == kFloat16) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(
         __builtin_bit_cast(half8_t, a.v[0]), __builtin_bit_cast(half8_t, b.v[0]), acc, 0, 0, 0);
@@ -172,10 +190,11 @@ template <int MS> __device__ __forceinline__ unsigned piece_y(int jj, int ii, in
   if constexpr (MS == kAcc16T) return jj * 16 + (lane >> 4) * 4 + ii;
   return MS == 16 ? jj * 16 + (lane & 15) : jj * 32 + (lane & 31);
 }
-template <int MS, typename Acc>
+// (TILE0: kAcc16T only, the first of the four tiles when a wave's tile rows hold more)
+template <int MS, int TILE0 = 0, typename Acc>
 __device__ __forceinline__ float piece_elem(const Acc &acc, int jj, int ii, int e) {
   if constexpr (MS == kAcc16T) {
-    return acc[jj][e][ii];
+    return acc[jj][TILE0 + e][ii];
   } else if constexpr (MS == 16) {
     return acc[jj][ii][e];
   } else {
@@ -842,7 +861,7 @@ __device__ __forceinline__ void mma_step32_interleaved(const char *slot, const i
 
 // Epilogue of one wave: alpha * acc + beta * C, conversion, bounds-checked
 // store, piece by piece (four consecutive elements of the contiguous C axis).
-template <int TOUT, int TX, int TY, int MS = 16, typename Acc>
+template <int TOUT, int TX, int TY, int MS = 16, int TILE0 = 0, typename Acc>
 __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned b, unsigned x_wave,
                                                 unsigned y_wave, int lane, const Acc &acc_re,
                                                 const Acc &acc_im) {
@@ -864,8 +883,8 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
       float re[4], im[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        re[e] = piece_elem<MS>(acc_re, j, i, e);
-        im[e] = piece_elem<MS>(acc_im, j, i, e);
+        re[e] = piece_elem<MS, TILE0>(acc_re, j, i, e);
+        im[e] = piece_elem<MS, TILE0>(acc_im, j, i, e);
         if (have_alpha) {
           const float r0 = re[e];
           re[e] = ar * r0 - ai * im[e];
@@ -1069,7 +1088,9 @@ __device__ __forceinline__ void store_wave_tile_rows(const KernelArgs &args, uns
                             : (have_alpha ? ai * re + ar * im : im);
         }
         Tout *p = out + (size_t)plane * nx * ny + (size_t)(j * 16 + e) * nx;
-        if constexpr (TOUT == kFloat32) {
+        if constexpr (kAblateStores) {
+          if (v[0] == 12345.678f) *p = (Tout)v[1];   // (timing-only build)
+        } else if constexpr (TOUT == kFloat32) {
           *reinterpret_cast<float4_t *>(p) = float4_t{v[0], v[1], v[2], v[3]};
         } else {
           Tout t[4] = {(Tout)v[0], (Tout)v[1], (Tout)v[2], (Tout)v[3]};
@@ -1408,7 +1429,11 @@ __device__ __attribute__((aligned(256))) char g_zero_tile[kTileBytes];
 
 template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+  if constexpr (kAblateBarrier) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+  }
 }
 
 // Both copy helpers write m0 (the LDS base of the copy) and say so in their
@@ -1418,6 +1443,7 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_offset,
                                                unsigned lds_address) {
+  if constexpr (kAblateCopies) return;
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
@@ -1431,6 +1457,7 @@ __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_o
 // are not contiguous in memory).
 __device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
                                                        unsigned lds_address) {
+  if constexpr (kAblateCopies) return;
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
@@ -1440,6 +1467,8 @@ __device__ __forceinline__ void load_1k_to_lds_by_lane(const char *lane_address,
       : "memory", "m0");
 }
 #pragma clang diagnostic pop
+
+#include "gemm_mfma_wide.h"
 
 template <int DT, int TOUT, int BX, int BY, int WX, int WY, int SLOTS, int WAVES_PER_EU, int LOADER,
           int MS, bool XT, int XSLOTS>
@@ -1955,6 +1984,23 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// The 192 x 256 block of gemm_mfma_wide.h (16-bit input, tiled layout): one
+// persistent block per compute unit.
+template <int DT, int TOUT>
+hipError_t launch_wide(const GemmParams &p, hipStream_t stream) {
+  const KernelArgs a = make_kernel_args(p, kWideBX, kWideBY);
+  const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
+  if (total == 0) return hipSuccess;
+  if (hipError_t e = check_grid(total)) return e;
+  auto kernel = complex_gemm_mfma_wide<DT, TOUT>;
+  static std::atomic<bool> lds_allowed[kMaxDevices];
+  if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
+  const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
+  const unsigned grid = (unsigned)(total < resident ? total : resident);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
+  return hipGetLastError();
+}
+
 // Whether 128 x 128 block tiles beat 256 x 128 ones for this problem: they do
 // when the larger tiles would leave compute units without work (fewer tiles
 // than units, or a last round that is mostly empty), although the smaller
@@ -1962,13 +2008,38 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
 // slower per flop it measured once every unit is busy). Estimated from the
 // fraction of unit-rounds that hold a tile under either tiling.
 inline bool small_tiles_pay(const GemmParams &p, double penalty) {
-  if (p.block_tile != 0) return p.block_tile == 2;
+  if (p.block_tile == 1 || p.block_tile == 2) return p.block_tile == 2;
   const size_t units = (size_t)compute_units();
   auto busy = [&](size_t bx, size_t by) {
     const size_t tiles = (size_t)p.batch * ceil_div((size_t)p.nx, bx) * ceil_div((size_t)p.ny, by);
     return (double)tiles / (double)(units * ceil_div(tiles, units));
   };
   return busy(128, 128) / penalty > busy(256, 128);
+}
+
+// Whether the 192 x 256 block of gemm_mfma_wide.h can compute this problem (what
+// its stores and its K loop assume), and whether it pays: per flop it measured
+// about 7 % faster than the 256 x 128 block once every compute unit is busy
+// (B=64 512x4096x576: 0.538 against 0.557 ms with 3 % of its tiles' columns
+// outside C), but its tiles are 1.5 times as large, so more of the last round of
+// tiles can stay empty (8192^3: 5.4 rounds of 192 x 256 tiles against 8 full ones).
+inline bool wide_tiles_apply(const GemmParams &p) {
+  return p.variant == kOpt && !p.input_interleaved && !p.c_interleaved && !p.have_alpha &&
+         !p.have_beta && ((uintptr_t)p.c % 16 == 0) && p.nx % 64 == 0 && p.ny % 64 == 0 &&
+         p.k_tiles >= 2 && !p.k_in_memory;
+}
+inline bool wide_tiles_pay(const GemmParams &p) {
+  if (p.block_tile != 0) return p.block_tile == 3;
+  const size_t units = (size_t)compute_units();
+  // fraction of the unit-rounds' tile area that holds elements of C
+  auto useful = [&](size_t bx, size_t by) {
+    const size_t cols = ceil_div((size_t)p.nx, bx), rows = ceil_div((size_t)p.ny, by);
+    const size_t tiles = (size_t)p.batch * cols * rows;
+    return (double)p.batch * p.nx * p.ny / (double)(units * ceil_div(tiles, units) * bx * by);
+  };
+  const double other = useful(256, 128) > useful(128, 128) / 1.15 ? useful(256, 128)
+                                                                   : useful(128, 128) / 1.15;
+  return useful(kWideBX, kWideBY) * 1.075 > other;
 }
 
 template <int DT, int TOUT>
@@ -1997,6 +2068,11 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     }
   }
   if (p.variant == kOpt || planar_direct) {
+    if constexpr (KPM == 1 && DtypeTraits<DT>::kElemBytes == 2) {
+      // 16-bit input, tiled operands, planar C with neither alpha nor beta: 192 x 256
+      // block, 4 waves of 192 x 64 (one per SIMD), where that pays
+      if (wide_tiles_apply(p) && wide_tiles_pay(p)) return launch_wide<DT, TOUT>(p, stream);
+    }
     if constexpr (KPM == 1) {
       // 16- and 32-bit input: 256 x 128 block, 8 waves of 64 x 64 (two per SIMD), 3-slot ring.
       // Interleaved fp32 C: in the exchanged-roles layout a lane's (re, im) pairs of

@@ -1,0 +1,521 @@
+// Wide-block variant of the direct-to-LDS complex GEMM for 16-bit input in the
+// tiled (opt) layout: a 192 x 256 patch of C per block, four waves (one per SIMD,
+// the whole register file each) of 192 x 64, i.e. 12 x 4 MFMA tiles of 16 x 16 and
+// 384 accumulator registers per lane.
+//
+// Compared with the 256 x 128 block of complex_gemm_mfma_dtl this moves 22 % fewer
+// bytes from L2 to LDS per flop (448 operand rows per 49152 products instead of
+// 384 per 32768), passes one barrier per 3072 instead of per 2048 matrix-core
+// cycles, and gives a K tile that much longer to arrive.
+//
+//  * One wave per SIMD has to keep the matrix core busy by itself: whatever else
+//    the wave issues goes between two matrix instructions, a few instructions at a
+//    time, and nothing may make it wait in the middle of the K loop.
+//  * X (the operand along the contiguous axis of C) is shared by the four waves:
+//    a ring of three 24 KiB slots in LDS, one barrier per K iteration. X is the
+//    instruction's "B" operand in the exchanged-roles layout of
+//    complex_gemm_mfma_dtl, so register e of four neighbouring tiles holds four
+//    consecutive x and C rows are stored straight from the accumulators.
+//  * Y is private: wave w multiplies rows 64 w .. 64 w + 63 of the block's Y and
+//    nobody else reads them, so the wave copies exactly those rows itself; its own
+//    s_waitcnt covers them and no barrier is involved. The wave holds the eight Y
+//    fragments of a K tile in registers for the whole iteration, so a Y slot is
+//    free as soon as they are read: two slots give the copy the same two
+//    iterations of lead as X has with three.
+//  * The iteration boundary lies inside the last X tile of an iteration: once the
+//    wave's last read of the current X slot has returned it waits for its copies
+//    of the next K tile, passes the barrier, and reads the next iteration's first
+//    X fragments and - each into the registers of its predecessor, right behind
+//    that one's last use - the next Y fragments, all behind the remaining matrix
+//    instructions of the tile. The next iteration starts with its operands in
+//    registers.
+//  * The order of a tile's 16 matrix instructions (two Y tile rows at a time) is
+//    chosen so that the Y fragments die one by one over the tile; for every sum it
+//    keeps the order of complex_gemm_mfma_dtl (Xr Yr before Xi Yi, Xr Yi before
+//    Xi Yr), so both kernels produce the same bits.
+//
+// Included by gemm_mfma.hip inside its namespaces, after the helpers it uses.
+#ifndef CCGLIB_AMD_GEMM_MFMA_WIDE_H_
+#define CCGLIB_AMD_GEMM_MFMA_WIDE_H_
+
+constexpr int kWideBX = 192, kWideBY = 256;
+constexpr int kWideXSlots = 3, kWideYSlots = 2;
+constexpr int kWideLdsBytes =
+    (kWideXSlots * 2 * kWideBX + kWideYSlots * 2 * kWideBY) * kTileRowBytes;   // 136 KiB
+constexpr int kWideTX = kWideBX / 16;   // X tiles of a wave
+
+// The MFMA as an inline-asm statement with the register file of the accumulator
+// spelled out. The compiler puts the accumulators of all matrix instructions of a
+// function into the AccVGPR half of the register file; with 384 of them it would
+// keep 128 in the other half and copy them in and out around every instruction
+// that uses them. Here the accumulators of the first eight X tiles are declared
+// as AccVGPRs (all 256) and those of the last four as ordinary VGPRs, and stay
+// where they are. What the compiler no longer does for these statements: the
+// wait states between a matrix instruction and a dependent read of its result by
+// another kind of instruction; the epilogue waits explicitly
+// (wait_for_mfma_results). A matrix instruction that adds to the result of the
+// one before needs none.
+// ZERO: the sum starts from zero (first K tile of a C tile).
+template <int DT, bool ACC_IN_AGPR, bool ZERO>
+__device__ __forceinline__ void mfma16_asm(float4_t &acc, const int4_t &a, const int4_t &b) {
+  if constexpr (kAblateMfma) {
+    // (timing-only build: the accumulator and the operands stay where they are)
+    if constexpr (ACC_IN_AGPR) {
+      asm volatile("" : "+a"(acc) : "v"(a), "v"(b));
+    } else {
+      asm volatile("" : "+v"(acc) : "v"(a), "v"(b));
+    }
+    return;
+  }
+#define CCGLIB_MFMA_ASM(OPCODE)                                                                    \
+  if constexpr (ACC_IN_AGPR) {                                                                     \
+    if constexpr (ZERO) {                                                                          \
+      asm volatile(OPCODE " %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));                          \
+    } else {                                                                                       \
+      asm volatile(OPCODE " %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));                         \
+    }                                                                                              \
+  } else {                                                                                         \
+    if constexpr (ZERO) {                                                                          \
+      asm volatile(OPCODE " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));                         \
+    } else {                                                                                       \
+      asm volatile(OPCODE " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));                         \
+    }                                                                                              \
+  }
+  if constexpr (DT == kFloat16) {
+    CCGLIB_MFMA_ASM("v_mfma_f32_16x16x32_f16")
+  } else {
+    static_assert(DT == kBfloat16, "16-bit input");
+    CCGLIB_MFMA_ASM("v_mfma_f32_16x16x32_bf16")
+  }
+#undef CCGLIB_MFMA_ASM
+}
+
+// Results of the matrix instructions issued last may be read by other instructions
+// only after up to 18 wait states.
+__device__ __forceinline__ void wait_for_mfma_results() {
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+}
+
+// Register e of the four tiles of a 64-column group are four consecutive x of a
+// C row: a lane writes 16 bytes (8 for fp16 / bf16 C) and a store instruction four
+// whole row segments, straight from the accumulators. This empty asm statement
+// takes four accumulators where they are at this point of the instruction stream.
+template <bool ACC_IN_AGPR>
+__device__ __forceinline__ void take_accumulators(float4_t &a, float4_t &b, float4_t &c, float4_t &d) {
+  if constexpr (ACC_IN_AGPR) {
+    asm volatile("" : "+a"(a), "+a"(b), "+a"(c), "+a"(d));
+  } else {
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+  }
+}
+
+// tile_coord for a tile id that differs from lane to lane (plain divisions).
+__device__ __forceinline__ TileCoord tile_coord_by_lane(const KernelArgs &args, unsigned wg) {
+  const unsigned per_batch = args.blocks_x * args.blocks_y;
+  const unsigned logical = xcd_remap(wg, per_batch * args.batch);
+  TileCoord tc;
+  tc.b = logical / per_batch;
+  const unsigned t = logical % per_batch;
+  constexpr unsigned GROUP = 4;
+  const unsigned group_size = GROUP * args.blocks_x;
+  const unsigned g = t / group_size, in_group = t % group_size;
+  const unsigned first_y = g * GROUP;
+  const unsigned rows_in_group = (args.blocks_y - first_y) < GROUP ? (args.blocks_y - first_y) : GROUP;
+  tc.block_y = first_y + in_group % rows_in_group;
+  tc.block_x = in_group / rows_in_group;
+  return tc;
+}
+
+
+template <int DT, int TOUT>
+__global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArgs args) {
+  static_assert(DtypeTraits<DT>::kTilesPerMfma == 1 && DtypeTraits<DT>::kElemBytes == 2,
+                "16-bit input");
+  constexpr int BX = kWideBX, BY = kWideBY, TX = kWideTX;
+  constexpr int XSLOTS = kWideXSlots, YSLOTS = kWideYSlots;
+  static_assert(XSLOTS == 3 && YSLOTS == 2, "both operands are requested two iterations ahead");
+  constexpr int XP = BX * kTileRowBytes, YP = BY * kTileRowBytes;   // one plane of a slot
+  constexpr int X_BYTES = 2 * XP, Y_BYTES = 2 * YP;
+  constexpr int Y_RING = XSLOTS * X_BYTES;
+  // 1 KiB copies a wave issues per K tile: 6 row blocks of X and its own 8 of Y
+  constexpr int kCopies = 14;
+  constexpr unsigned GROUP = 64 * kTileRowBytes;   // 64 rows of a slot
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const unsigned k_tiles = args.k_tiles;
+  const unsigned total = args.blocks_x * args.blocks_y * args.batch;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
+
+  // ---- the C tiles of this block -------------------------------------------------
+  // Tile n of the block is C tile blockIdx.x + n gridDim.x. Lane n works out the
+  // coordinates of tile n once (the first 64; a block with more takes the slow
+  // way for the rest), and the wave fetches them with a lane read at every tile
+  // change: with one wave per SIMD the divisions would otherwise stand in the
+  // middle of the MFMA stream.
+  const unsigned my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  unsigned table_b, table_x, table_y;
+  {
+    unsigned vt = blockIdx.x + (unsigned)lane * gridDim.x;
+    vt = vt < total ? vt : blockIdx.x;
+    const TileCoord tc = tile_coord_by_lane(args, vt);
+    table_b = tc.b;
+    table_x = tc.block_x;
+    table_y = tc.block_y;
+  }
+  auto coords = [&](unsigned n) {   // past the last tile: the last one again (copied, never used)
+    n = n < my_tiles ? n : my_tiles - 1;
+    TileCoord tc;
+    if (n < 64) {
+      tc.b = (unsigned)__builtin_amdgcn_readlane((int)table_b, (int)n);
+      tc.block_x = (unsigned)__builtin_amdgcn_readlane((int)table_x, (int)n);
+      tc.block_y = (unsigned)__builtin_amdgcn_readlane((int)table_y, (int)n);
+    } else {
+      tc = tile_coord(args, blockIdx.x + n * gridDim.x);
+    }
+    return tc;
+  };
+
+  // ---- the copy --------------------------------------------------------------
+  // What a lane fetches of a 1 KiB row block (16 rows x 64 bytes) so that the
+  // hardware's linear write (lane L at 16 L) produces the swizzled LDS layout:
+  // Y: chunk XOR (row >> 1) & 3; X: the exchanged-roles order of rows and chunks,
+  // whose chunk XOR depends on the parity of the row block
+  // (see complex_gemm_mfma_dtl).
+  const unsigned lane_off_y = (lane >> 2) * kTileRowBytes + (((lane & 3) ^ ((lane >> 3) & 3)) * 16);
+  const int xt_row = 4 * (lane >> 4) + (((lane >> 2) & 3) ^ (lane >> 4));
+  const unsigned lane_off_x_even = xt_row * kTileRowBytes + (lane & 3) * 16;
+  const unsigned lane_off_x_odd = xt_row * kTileRowBytes + ((lane & 3) ^ 3) * 16;
+
+  // Wave w copies the row blocks 6 (w & 1) .. + 5 of plane w / 2 of X (consecutive
+  // KiB of the slot) and the 64 rows of Y that it multiplies (4 consecutive KiB in
+  // either plane).
+  const unsigned x_plane = wave >> 1, x_rb0 = 6 * (wave & 1);
+  const unsigned x_lds = lds_base + x_plane * XP + x_rb0 * 1024;
+  const unsigned y_lds = lds_base + Y_RING + wave * 64 * kTileRowBytes;
+  struct Stream {
+    unsigned n, kt;   // tile of the block and K tile of the request issued last
+  };
+  Stream xs{0, 0}, ys{0, 0};
+  // wave-uniform: K tile 0 of the operand tile that holds row block i of the wave's
+  // six of X; K tile 0 of the wave's rows of Y (re plane)
+  const char *x_src[6], *y_src = nullptr;
+  auto point_x = [&](unsigned n) {
+    const TileCoord tc = coords(n);
+    const char *op = args.x + (size_t)tc.b * args.x_batch_bytes + x_plane * kTilePlaneBytes;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      const unsigned row0 = tc.block_x * BX + (x_rb0 + i) * 16;
+      unsigned tile = row0 / kTileRows;
+      tile = tile < args.x_tiles ? tile : args.x_tiles - 1;   // rows past the end: never stored
+      x_src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes +
+                 (row0 % kTileRows) * kTileRowBytes;
+    }
+  };
+  auto point_y = [&](unsigned n) {
+    const TileCoord tc = coords(n);
+    const unsigned row0 = tc.block_y * BY + wave * 64;
+    unsigned tile = row0 / kTileRows;
+    tile = tile < args.y_tiles ? tile : args.y_tiles - 1;
+    y_src = args.y + (size_t)tc.b * args.y_batch_bytes +
+            (size_t)tile * args.k_tile_stride * kTileBytes + (row0 % kTileRows) * kTileRowBytes;
+  };
+  // Copy c of the 14 of a K tile: 0 - 7 the wave's rows of Y (re plane, then im),
+  // 8 - 13 its row blocks of X. One at a time and well apart: every vector memory
+  // instruction occupies the compute unit's address unit for 16 cycles, and a wave
+  // that issues the next one earlier waits - with its matrix instructions behind it.
+  auto issue = [&](int c, unsigned x_slot, unsigned y_slot) {
+    if (c < 8) {
+      const int plane = c >> 2, blk = c & 3;
+      load_1k_to_lds(y_src + (size_t)ys.kt * kTileBytes + plane * kTilePlaneBytes + blk * 1024,
+                     lane_off_y, y_lds + y_slot * Y_BYTES + plane * YP + blk * 1024);
+    } else {
+      const int i = c - 8;
+      load_1k_to_lds(x_src[i] + (size_t)xs.kt * kTileBytes, (i & 1) ? lane_off_x_odd : lane_off_x_even,
+                     x_lds + x_slot * X_BYTES + i * 1024);
+    }
+  };
+  auto advance_x = [&] {
+    if (++xs.kt == k_tiles) {
+      xs.kt = 0;
+      point_x(++xs.n);
+    }
+  };
+  auto advance_y = [&] {
+    if (++ys.kt == k_tiles) {
+      ys.kt = 0;
+      point_y(++ys.n);
+    }
+  };
+
+  // ---- fragments ---------------------------------------------------------------
+  typedef __attribute__((address_space(3))) const int4_t lds_int4_t;
+  auto rd = [](unsigned address) { return *reinterpret_cast<lds_int4_t *>(address); };
+  const int r16 = lane & 15, g4 = lane >> 4;
+  unsigned xo[4];   // X fragment of tile i of a 64-row group, inside a slot
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    xo[i] = lds_base + (4 * r16 + (i ^ (r16 & 3))) * kTileRowBytes +
+            ((g4 ^ (3 * ((r16 >> 2) & 1))) * 16);
+  }
+  const unsigned yo = y_lds + swizzled_row_offset(r16, g4);
+
+  // ---- pipeline ------------------------------------------------------------------
+  point_x(0);
+  point_y(0);
+  // the requests that iterations -2 and -1 would have made
+#pragma unroll
+  for (int c = 0; c < kCopies; ++c) issue(c, 0, 0);
+  advance_y();
+  advance_x();
+#pragma unroll
+  for (int c = 0; c < kCopies; ++c) issue(c, 1, 1);
+
+  unsigned x_slot = 0, y_slot = 0;   // slots of the current iteration
+  int4_t yr[4], yi[4];               // the Y fragments of the current K tile
+  int4_t xr[2], xi[2], xn[2];        // X fragments (re, im, -im) of the current and the next tile
+  auto flip = [](const int4_t &v) {
+    int4_t o;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) o[w] = v[w] ^ (int)DtypeTraits<DT>::kSignMask;
+    return o;
+  };
+  // what the last tile of "iteration -1" would have done for iteration 0
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies) : "memory");
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    yr[j] = rd(yo + j * 16 * kTileRowBytes);
+    yi[j] = rd(yo + YP + j * 16 * kTileRowBytes);
+  }
+  if constexpr (!kAblateBarrier) asm volatile("s_barrier" ::: "memory");
+  xr[0] = rd(xo[0]);
+  xi[0] = rd(xo[0] + XP);
+  xn[0] = flip(xi[0]);
+
+  float4_t acc_re[4][TX], acc_im[4][TX];
+
+  // ---- the C stores ----------------------------------------------------------------
+  // A wave's 192 x 64 patch leaves in 96 store instructions of four 256-byte row
+  // segments (see store_piece), none of them after the K loop: they are issued one
+  // every other matrix instruction behind those of the tile's LAST K iteration and
+  // of the next tile's FIRST one, as the accumulators become final and before they
+  // are started again:
+  //   group 0 (X tiles 0 - 3, final behind tile 3 of the last iteration): last iteration;
+  //   group 1 (tiles 4 - 7): half in the last iteration, half in the next first one
+  //   (which starts these accumulators again with its tile 4);
+  //   group 2 (tiles 8 - 11): the next first iteration, before its tile 8.
+  // The host only launches this kernel for planar C without alpha and beta, with
+  // 16-byte aligned rows and nx, ny multiples of 64: a 64 x 64 piece of a tile is
+  // either inside C or outside.
+  using Tout = typename OutType<TOUT>::type;
+  struct StoreTarget {
+    char *base;        // wave-uniform: row y_wave, column x_block of the tile's re plane
+    bool inside[3];    // the wave's rows and the group's columns are inside C
+    bool all;          // all three: every store of the tile is issued
+  };
+  StoreTarget target{nullptr, {false, false, false}, false};
+  const unsigned lane_store_off =
+      (unsigned)((((lane >> 4) * 4) * (size_t)args.nx + (lane & 15) * 4) * sizeof(Tout));
+  const size_t plane_bytes = (size_t)args.nx * args.ny * sizeof(Tout);
+  auto aim_stores = [&](unsigned n) {
+    const TileCoord tc = coords(n);
+    const unsigned x_block = tc.block_x * BX, y_wave = tc.block_y * BY + wave * 64;
+    target.base = args.c + ((size_t)tc.b * 2 * args.nx * args.ny + (size_t)y_wave * args.nx + x_block) *
+                               sizeof(Tout);
+    const bool y_in = y_wave < args.ny;
+    target.inside[0] = y_in;
+    target.inside[1] = y_in && x_block + 64 < args.nx;
+    target.inside[2] = y_in && x_block + 128 < args.nx;
+    target.all = target.inside[2];
+  };
+  // Store s (0 .. 31) of group g: tile row j = s / 8, plane (s / 4) % 2, register e =
+  // s % 4 of the group's four tiles, which are four consecutive x of row 16 j + 4
+  // (lane / 16) + e. The empty asm statement takes the accumulators where they are,
+  // here and now: without it the compiler may read them right behind the matrix
+  // instruction that wrote them, whose wait states it does not know.
+  auto store_piece = [&](int g, int s) {
+    if (!target.inside[g]) return;
+    const int j = s >> 3, plane = (s >> 2) & 1, e = s & 3;
+    float4_t(&acc)[4][TX] = plane == 0 ? acc_re : acc_im;
+    if (g < 2) {
+      take_accumulators<true>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+    } else {
+      take_accumulators<false>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+    }
+    const float v[4] = {acc[j][4 * g][e], acc[j][4 * g + 1][e], acc[j][4 * g + 2][e],
+                        acc[j][4 * g + 3][e]};
+    char *p = target.base + plane * plane_bytes +
+              ((size_t)(j * 16 + e) * args.nx + g * 64) * sizeof(Tout) + lane_store_off;
+    if constexpr (kAblateStores) {
+      if (v[0] == 12345.678f) *reinterpret_cast<Tout *>(p) = (Tout)v[1];   // (timing-only build)
+    } else if constexpr (TOUT == kFloat32) {
+      *reinterpret_cast<float4_t *>(p) = float4_t{v[0], v[1], v[2], v[3]};
+    } else {
+      Tout t4[4] = {(Tout)v[0], (Tout)v[1], (Tout)v[2], (Tout)v[3]};
+      *reinterpret_cast<ushort4_t *>(p) = __builtin_bit_cast(ushort4_t, t4);
+    }
+  };
+  constexpr int kStoresPerIteration = 48;
+
+  // One K iteration. `first`: the first one of a C tile (sums start from zero);
+  // written out on its own, so that the accumulators have one definition there and
+  // one chain of updates in the loop over the middle ones. `carry`: a first
+  // iteration that issues the remaining stores of the previous C tile. `last`:
+  // the last one of a C tile, which issues the first half of its stores.
+  auto iteration = [&](auto first, auto carry, auto last) {
+    constexpr bool FIRST = decltype(first)::value, CARRY = decltype(carry)::value,
+                   LAST = decltype(last)::value;
+    // the bookkeeping (which branches at a C tile change) of the copies issued
+    // inside this iteration: K tile + 2 of both operands
+    advance_y();
+    advance_x();
+    const unsigned x_next = x_slot + 1 == XSLOTS ? 0 : x_slot + 1;
+    const unsigned x_refill = x_slot >= 1 ? x_slot - 1 : XSLOTS - 1;   // (x_slot + 2) % 3
+    const unsigned xa = x_slot * X_BYTES, xa_next = x_next * X_BYTES;
+    const unsigned ya_next = yo + (y_slot ^ 1) * Y_BYTES;
+#define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
+    // what else is issued behind MFMA p of tile t
+    auto behind = [&](int t, int p) {
+      const int s = t & 1;
+      if (t + 1 < TX) {
+        // the next tile's X fragments into the other register set
+        if (p == 0) {
+          const unsigned a = xo[(t + 1) & 3] + xa + ((t + 1) >> 2) * GROUP;
+          xr[s ^ 1] = rd(a);
+          xi[s ^ 1] = rd(a + XP);
+          CCGLIB_PIN;
+        }
+        if (p >= 10 && p < 14) {
+          // -im of the next tile, one instruction behind each of four MFMAs (four in a
+          // row would hold up the next MFMA); pinned on both sides: moved up, it
+          // would wait for the read just issued
+          CCGLIB_PIN;
+          xn[s ^ 1][p - 10] = xi[s ^ 1][p - 10] ^ (int)DtypeTraits<DT>::kSignMask;
+          CCGLIB_PIN;
+        }
+      }
+      {
+        // C stores behind every other MFMA (the odd ones; the copies go behind even
+        // ones), all of them before the last copy of the iteration
+        const int idx = 16 * t + p;
+        if (LAST && (idx & 1) && idx >= 65 && idx < 65 + 2 * kStoresPerIteration) {
+          const int s = (idx - 65) / 2;
+          store_piece(s < 32 ? 0 : 1, s < 32 ? s : s - 32);
+          CCGLIB_PIN;
+        }
+        if (CARRY && (idx & 1) && idx < 1 + 2 * kStoresPerIteration) {
+          const int s = (idx - 1) / 2;
+          store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+          CCGLIB_PIN;
+        }
+      }
+      {
+        // The copy of K tile + 2, one instruction every 12 MFMAs from tile 1 on: the
+        // Y slot whose fragments this iteration holds in registers, and the X slot
+        // that the barrier of the previous iteration's last tile released.
+        const int m = 16 * t + p - 16;
+        if (m >= 0 && m % 12 == 6 && m / 12 < kCopies) {
+          issue(m / 12, x_refill, y_slot);
+          CCGLIB_PIN;
+        }
+      }
+      if (t == TX - 1) {
+        // The iteration boundary. MFMA 4 of the last tile has waited for the
+        // wave's last fragment read from this X slot.
+        if (p == 4) {
+          // This wave's copies of the next K tile are complete when nothing older
+          // than the requests of this iteration is outstanding - which are its
+          // copies and, in a first or last iteration of a tile that lies entirely
+          // inside C, its 48 stores (the counter retires loads in order and does
+          // not tell them from stores; where stores may have been skipped, the
+          // smaller number is the safe one and waits for more than it has to).
+          if ((CARRY || LAST) && target.all) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies + kStoresPerIteration) : "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies) : "memory");
+          }
+          // every wave's part of the next X tile has landed, and nobody reads the
+          // current X slot any more
+          if constexpr (!kAblateBarrier) asm volatile("s_barrier" ::: "memory");
+          xr[0] = rd(xo[0] + xa_next);
+          xi[0] = rd(xo[0] + xa_next + XP);
+          yr[0] = rd(ya_next);
+          CCGLIB_PIN;
+        }
+        // each Y fragment of the next K tile into the registers of its
+        // predecessor, behind that one's last use
+        if (p == 5) yr[1] = rd(ya_next + 16 * kTileRowBytes);
+        if (p == 6) yi[0] = rd(ya_next + YP);
+        if (p == 7) yi[1] = rd(ya_next + YP + 16 * kTileRowBytes);
+        if (p == 12) yr[2] = rd(ya_next + 32 * kTileRowBytes);
+        if (p == 13) yr[3] = rd(ya_next + 48 * kTileRowBytes);
+        if (p == 14) yi[2] = rd(ya_next + YP + 32 * kTileRowBytes);
+        if (p == 15) yi[3] = rd(ya_next + YP + 48 * kTileRowBytes);
+        if (p >= 5) CCGLIB_PIN;
+        if (p >= 12) {
+          xn[0][p - 12] = xi[0][p - 12] ^ (int)DtypeTraits<DT>::kSignMask;
+          CCGLIB_PIN;
+        }
+      }
+    };
+#pragma unroll
+    for (int t = 0; t < TX; ++t) {
+      const int s = t & 1;
+      // exchanged roles: Y supplies the instruction's "A" rows, X its "B" columns
+#define CCGLIB_MM(ACC, Y, X, Z, P)                                                     \
+  if (t < 8) {                                                                         \
+    mfma16_asm<DT, true, Z>(ACC, Y, X);                                                \
+  } else {                                                                             \
+    mfma16_asm<DT, false, Z>(ACC, Y, X);                                               \
+  }                                                                                    \
+  behind(t, P);
+      CCGLIB_MM(acc_re[0][t], yr[0], xr[s], FIRST, 0)
+      CCGLIB_MM(acc_re[1][t], yr[1], xr[s], FIRST, 1)
+      CCGLIB_MM(acc_im[0][t], yi[0], xr[s], FIRST, 2)
+      CCGLIB_MM(acc_im[1][t], yi[1], xr[s], FIRST, 3)
+      CCGLIB_MM(acc_im[0][t], yr[0], xi[s], false, 4)
+      CCGLIB_MM(acc_im[1][t], yr[1], xi[s], false, 5)
+      CCGLIB_MM(acc_re[0][t], yi[0], xn[s], false, 6)
+      CCGLIB_MM(acc_re[1][t], yi[1], xn[s], false, 7)
+      CCGLIB_MM(acc_re[2][t], yr[2], xr[s], FIRST, 8)
+      CCGLIB_MM(acc_re[3][t], yr[3], xr[s], FIRST, 9)
+      CCGLIB_MM(acc_im[2][t], yi[2], xr[s], FIRST, 10)
+      CCGLIB_MM(acc_im[3][t], yi[3], xr[s], FIRST, 11)
+      CCGLIB_MM(acc_im[2][t], yr[2], xi[s], false, 12)
+      CCGLIB_MM(acc_im[3][t], yr[3], xi[s], false, 13)
+      CCGLIB_MM(acc_re[2][t], yi[2], xn[s], false, 14)
+      CCGLIB_MM(acc_re[3][t], yi[3], xn[s], false, 15)
+#undef CCGLIB_MM
+    }
+#undef CCGLIB_PIN
+    x_slot = x_next;
+    y_slot ^= 1;
+  };
+
+  // (k_tiles >= 2: the host does not launch this kernel for a K of one tile)
+  using Yes = std::true_type;
+  using No = std::false_type;
+  for (unsigned n = 0; n < my_tiles; ++n) {
+    if (n == 0) {
+      iteration(Yes{}, No{}, No{});
+    } else {
+      iteration(Yes{}, Yes{}, No{});
+    }
+    for (unsigned it = 2; it < k_tiles; ++it) iteration(No{}, No{}, No{});
+    aim_stores(n);
+    iteration(No{}, No{}, Yes{});
+  }
+  // the second half of the last tile's stores
+  wait_for_mfma_results();
+#pragma unroll
+  for (int s = 0; s < kStoresPerIteration; ++s) {
+    store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // nothing may still be writing into LDS when the block gives it back
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+#endif  // CCGLIB_AMD_GEMM_MFMA_WIDE_H_

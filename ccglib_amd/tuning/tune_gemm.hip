@@ -1,19 +1,35 @@
-// Offline sweep over kernel configurations of the tiled-input complex GEMM on
-// one gfx950 device: the counterpart of the reference's tuning/tune_gemm.py
-// (which sweeps block and warp tile sizes of its kernel through a JIT tuner).
+// Offline sweep over kernel configurations of the complex GEMM on one gfx950
+// device: the counterpart of the reference's tuning/tune_gemm.py (which sweeps
+// block and warp tile sizes of its kernel through a JIT tuner).
 // The configurations here are template instantiations of the library's own
-// kernel (block tile, wave tile, ring slots, MFMA shape), timed back to back on
-// random operands of the given shape; the library's dispatch
+// kernels (block tile, wave tile, ring slots, MFMA shape, operand layout), timed
+// back to back on operands of the given shape; the library's dispatch
 // (launch_typed in ../csrc/gemm_mfma.hip) uses the winners.
 //
-//   make && ./tune_gemm [B M N K [filter]]       e.g.  ./tune_gemm 64 512 4096 576 f16
-//   ZERO=1 ./tune_gemm ...                       all-zero operands (no power limit)
+//   make && ./tune_gemm [--fill=baseline|legacy|zero] [B M N K [filter]]
+//                                            e.g.  ./tune_gemm 64 512 4096 576 f16
+//
+// --fill=baseline (default): the operand distributions of the benchmark
+//   configurations - real and imaginary parts N(0, 1) for fp16 / bf16 / fp32
+//   (for B=64 M=512 N=4096 K=576, the beamformer shape, the M-row operand holds
+//   unit-magnitude random phases), N(0, 1) scaled into the fp8 range (x 448 / 5.8
+//   for e4m3: the largest of 10^8 normal samples is about 5.8) and quantised,
+//   Bernoulli(0.5) bits for 1-bit input. The part is power limited, and what the
+//   operands hold decides how fast a kernel runs.
+// --fill=legacy: the fill of earlier sweeps (a 2 MiB pattern of numbers with three
+//   exponents; fp8 without sign bit), kept for comparison with their files.
+// --fill=zero: all-zero operands (no power limit).
+// `make ABLATE=n` builds timing-only variants (see CCGLIB_ABLATE in gemm_mfma.hip).
 #include "../csrc/gemm_mfma.hip"
+#include "../csrc/gemm_int1.hip"
+
+#include <hip/hip_fp8.h>
 
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <string>
 #include <vector>
 
 using namespace ccglib_amd;
@@ -33,24 +49,40 @@ struct Config {
   LaunchFn launch;
   int type_in, type_out;
   int layout = kLoadTiled;   // operand layout the configuration reads
+  double peak = 0;           // what "of peak" refers to (0: the input type's MFMA peak)
 };
 
-// name: type, block BX x BY, wave WX x WY, ring slots, MFMA rows
+// the 1-bit GEMM on the vector ALUs (XOR + population count), whatever the layout
+static hipError_t launch_popcount(const GemmParams &p, hipStream_t stream) {
+  GemmParams q = p;
+  q.int1_direct = 0;
+  return launch_gemm_int1(q, stream);
+}
+// 256 CUs x 64 lane-operations per clock x 2.4 GHz, 8 lane-operations (4 XOR, 4
+// counts) per 32 complex products of 8 "operations" each
+constexpr double kPopcountRoof = 256 * 64 * 2.4e9 * 32 / 1e12;   // 1258 TOP/s
+
+// name: type, [operand layout,] block BX x BY, wave WX x WY, ring slots, MFMA rows
 static const std::vector<Config> kConfigs = {
     {"f16 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"f16 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 y3 x4 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true, 4>, kFloat16, kFloat32},
+    {"f16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32>, kFloat16, kFloat32},
     {"f16 256x128 w64x64 s3 m32", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat16, kFloat32},
     {"f16 128x128 w64x64 s2 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"f16 128x128 w64x32 s4 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat16, kFloat32},
-    {"bf16 256x128 w64x64 s3 m16", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kBfloat16, kFloat32},
+    {"bf16 256x128 w64x64 s3 m16 xt", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kBfloat16, kFloat32},
+    {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32>, kBfloat16, kFloat32},
     {"f32 256x128 w64x64 s3 m16", launch_dtl<kFloat32, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat32, kFloat32},
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"fp8 128x128 w64x64 s2 m32", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"fp8 128x128 w64x32 s4 m32", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"int1 128x128 w64x64 s2 m32", launch_dtl<kInt1, kInt32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>, kInt1, kInt32},
     {"int1 256x128 w64x64 s3 m32", launch_dtl<kInt1, kInt32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kInt1, kInt32},
+    // the 1-bit GEMM on the vector ALUs; "of peak" is of its issue roof
+    {"int1 popcount 128x128 (vector ALU)", launch_popcount, kInt1, kInt32, kLoadTiled, kPopcountRoof},
+    {"int1 popcount planar 128x128 (vector ALU)", launch_popcount, kInt1, kInt32, kLoadPlanarVec, kPopcountRoof},
     // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
     {"f16 planar 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>, kFloat16, kFloat32, kLoadPlanarVec},
@@ -69,8 +101,94 @@ static double peak_of(int type) {
   }
 }
 
-// Random operand bytes that are ordinary numbers in the given type.
-static void fill(std::vector<unsigned short> &h, int type) {
+// ---- operand fills ----------------------------------------------------------------
+// A counter-based generator: what an element holds depends on its index and the
+// seed only.
+__device__ __forceinline__ unsigned mix32(unsigned long long x) {
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdull;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ull;
+  x ^= x >> 33;
+  return (unsigned)x;
+}
+__device__ __forceinline__ float uniform01(unsigned r) { return (r >> 8) * (1.0f / 16777216.0f) + 0x1p-25f; }
+
+template <typename T> __device__ __forceinline__ T to_type(float v);
+template <> __device__ __forceinline__ _Float16 to_type<_Float16>(float v) { return (_Float16)v; }
+template <> __device__ __forceinline__ __bf16 to_type<__bf16>(float v) { return (__bf16)v; }
+template <> __device__ __forceinline__ float to_type<float>(float v) { return v; }
+template <> __device__ __forceinline__ unsigned char to_type<unsigned char>(float v) {
+  // e4m3, saturating, round to nearest even; N(0, 1) scaled into the type's range
+  return (unsigned char)__hip_cvt_float_to_fp8(v * (448.0f / 5.8f), __HIP_SATFINITE, __HIP_E4M3);
+}
+
+// Pair i of an operand is the (re, im) of one complex element; `pos` maps it to
+// the two element offsets of the layout in use. PHASES: unit magnitude, random
+// phase; otherwise both parts N(0, 1).
+struct PairLayout {
+  int layout;
+  unsigned long long plane;   // tiled: elements of one tile plane; planar: of one operand plane
+};
+template <typename T, bool PHASES>
+__global__ void fill_pairs(T *out, unsigned long long pairs, PairLayout pl, unsigned long long seed) {
+  for (unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x; i < pairs;
+       i += (unsigned long long)gridDim.x * blockDim.x) {
+    const float u = uniform01(mix32(2 * i + seed)), w = uniform01(mix32(2 * i + 1 + seed));
+    const float angle = 6.2831853f * w;
+    const float radius = PHASES ? 1.0f : sqrtf(-2.0f * logf(u));
+    const float re = radius * cosf(angle), im = radius * sinf(angle);
+    unsigned long long ire, iim;
+    if (pl.layout == kLoadInterleavedVec) {
+      ire = 2 * i;
+      iim = 2 * i + 1;
+    } else {   // a re plane followed by an im plane, per tile or per batch
+      ire = (i / pl.plane) * 2 * pl.plane + i % pl.plane;
+      iim = ire + pl.plane;
+    }
+    out[ire] = to_type<T>(re);
+    out[iim] = to_type<T>(im);
+  }
+}
+__global__ void fill_words(unsigned *out, unsigned long long words, unsigned long long seed) {
+  for (unsigned long long i = blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x; i < words;
+       i += (unsigned long long)gridDim.x * blockDim.x) {
+    out[i] = mix32(i + seed);
+  }
+}
+
+static void fill_baseline(void *d, size_t bytes, int type, int layout, size_t plane_elems, bool phases,
+                          unsigned long long seed) {
+  const dim3 grid(4096), block(256);
+  if (type == kInt1) {
+    hipLaunchKernelGGL(fill_words, grid, block, 0, 0, (unsigned *)d, (unsigned long long)(bytes / 4), seed);
+    return;
+  }
+  const size_t elem = (size_t)bits_of(type) / 8;
+  const unsigned long long pairs = bytes / elem / 2;
+  const PairLayout pl{layout, (unsigned long long)plane_elems};
+#define FILL(T)                                                                                     \
+  if (phases) {                                                                                     \
+    hipLaunchKernelGGL((fill_pairs<T, true>), grid, block, 0, 0, (T *)d, pairs, pl, seed);           \
+  } else {                                                                                          \
+    hipLaunchKernelGGL((fill_pairs<T, false>), grid, block, 0, 0, (T *)d, pairs, pl, seed);          \
+  }
+  if (type == kFloat16) {
+    FILL(_Float16)
+  } else if (type == kBfloat16) {
+    FILL(__bf16)
+  } else if (type == kFloat32) {
+    FILL(float)
+  } else {
+    FILL(unsigned char)
+  }
+#undef FILL
+}
+
+// The fill of earlier sweeps: random operand bytes that are ordinary numbers in the
+// given type, a 2 MiB pattern repeated over the operand.
+static void fill_legacy(void *d, size_t bytes, int type) {
+  std::vector<unsigned short> h(1 << 20);
   std::srand(1);
   for (auto &v : h) {
     const unsigned r = (unsigned)std::rand();
@@ -87,22 +205,39 @@ static void fill(std::vector<unsigned short> &h, int type) {
     float *f = reinterpret_cast<float *>(h.data());
     for (size_t i = 0; i < h.size() / 2; ++i) f[i] = (std::rand() / (float)RAND_MAX) * 4.f - 2.f;
   }
+  for (size_t o = 0; o < bytes; o += h.size() * 2)
+    CHECK(hipMemcpy((char *)d + o, h.data(), std::min(h.size() * 2, bytes - o), hipMemcpyHostToDevice));
 }
 
 int main(int argc, char **argv) {
   unsigned B = 64, M = 512, N = 4096, K = 576;
-  if (argc > 4) {
-    B = (unsigned)std::atoi(argv[1]);
-    M = (unsigned)std::atoi(argv[2]);
-    N = (unsigned)std::atoi(argv[3]);
-    K = (unsigned)std::atoi(argv[4]);
+  std::string fill = std::getenv("ZERO") ? "zero" : "baseline";
+  std::vector<const char *> pos;
+  for (int i = 1; i < argc; ++i) {
+    if (std::strncmp(argv[i], "--fill=", 7) == 0) {
+      fill = argv[i] + 7;
+    } else {
+      pos.push_back(argv[i]);
+    }
   }
-  const char *filter = argc > 5 ? argv[5] : (argc == 2 ? argv[1] : nullptr);
+  if (fill != "baseline" && fill != "legacy" && fill != "zero") {
+    std::printf("unknown fill '%s' (baseline, legacy or zero)\n", fill.c_str());
+    return 1;
+  }
+  if (pos.size() >= 4) {
+    B = (unsigned)std::atoi(pos[0]);
+    M = (unsigned)std::atoi(pos[1]);
+    N = (unsigned)std::atoi(pos[2]);
+    K = (unsigned)std::atoi(pos[3]);
+  }
+  const char *filter = pos.size() > 4 ? pos[4] : (pos.size() == 1 ? pos[0] : nullptr);
+  const bool beamformer = B == 64 && M == 512 && N == 4096 && K == 576;
   hipEvent_t e0, e1;
   CHECK(hipEventCreate(&e0));
   CHECK(hipEventCreate(&e1));
-  std::printf("%-40s %10s %12s %10s   (B=%u M=%u N=%u K=%u%s)\n", "configuration", "ms", "TFLOP/s", "of peak", B, M, N, K,
-              std::getenv("ZERO") ? ", zero operands" : "");
+  std::printf("%-44s %10s %12s %10s   (B=%u M=%u N=%u K=%u, %s operands%s)\n", "configuration", "ms", "TFLOP/s",
+              "of peak", B, M, N, K, fill.c_str(), CCGLIB_ABLATE ? ", TIMING-ONLY BUILD" : "");
+  if (CCGLIB_ABLATE) std::printf("CCGLIB_ABLATE = %d: parts of the kernels are left out, C is wrong\n", CCGLIB_ABLATE);
   for (const Config &c : kConfigs) {
     if (filter && !std::strstr(c.name, filter)) continue;
     GemmParams p;
@@ -125,6 +260,12 @@ int main(int argc, char **argv) {
     p.beta_im = 0;
     p.have_alpha = 0;
     p.have_beta = 0;
+    if (c.launch == launch_wide<kFloat16, kFloat32> || c.launch == launch_wide<kBfloat16, kFloat32>) {
+      if (!wide_tiles_apply(p)) {
+        std::printf("%-44s (not applicable to this shape)\n", c.name);
+        continue;
+      }
+    }
     // whole tiles: at least as large as the planar and interleaved layouts
     const unsigned k_tiles_planar = (K + kpt - 1) / kpt;
     const size_t x_bytes = (size_t)B * p.x_tiles * k_tiles_planar * kTileBytes;
@@ -134,15 +275,21 @@ int main(int argc, char **argv) {
     CHECK(hipMalloc(&dx, x_bytes));
     CHECK(hipMalloc(&dy, y_bytes));
     CHECK(hipMalloc(&dc, c_bytes));
-    std::vector<unsigned short> h(1 << 20);
-    fill(h, c.type_in);
-    for (size_t o = 0; o < x_bytes; o += h.size() * 2)
-      CHECK(hipMemcpy((char *)dx + o, h.data(), std::min(h.size() * 2, x_bytes - o), hipMemcpyHostToDevice));
-    for (size_t o = 0; o < y_bytes; o += h.size() * 2)
-      CHECK(hipMemcpy((char *)dy + o, h.data(), std::min(h.size() * 2, y_bytes - o), hipMemcpyHostToDevice));
-    if (std::getenv("ZERO")) {
+    if (fill == "zero") {
       CHECK(hipMemset(dx, 0, x_bytes));
       CHECK(hipMemset(dy, 0, y_bytes));
+    } else if (fill == "legacy") {
+      fill_legacy(dx, x_bytes, c.type_in);
+      fill_legacy(dy, y_bytes, c.type_in);
+    } else {
+      // elements of one plane: of a tile (tiled layout) or of one batch's operand plane
+      const size_t elem_bits = (size_t)bits_of(c.type_in);
+      const size_t tile_plane = (size_t)kTilePlaneBytes * 8 / elem_bits;
+      const size_t xp = c.layout == kLoadTiled ? tile_plane : (size_t)N * K;
+      const size_t yp = c.layout == kLoadTiled ? tile_plane : (size_t)M * K;
+      fill_baseline(dx, x_bytes, c.type_in, c.layout, xp, false, 1);
+      fill_baseline(dy, y_bytes, c.type_in, c.layout, yp, beamformer && c.type_in != kInt1, 2);
+      CHECK(hipDeviceSynchronize());
     }
     p.x = dx;
     p.y = dy;
@@ -168,13 +315,13 @@ int main(int argc, char **argv) {
     best /= iters;
     const double tflops = 8.0 * B * M * N * K / (best * 1e-3) / 1e12;
     // a hash of C's bits: configurations that multiply the same operands in the same
-    // layout with the same MFMA shape must agree
+    // layout must agree
     std::vector<unsigned> hc(c_bytes / 4);
     CHECK(hipMemcpy(hc.data(), dc, c_bytes, hipMemcpyDeviceToHost));
     unsigned long long hash = 1469598103934665603ull;
     for (unsigned v : hc) hash = (hash ^ v) * 1099511628211ull;
-    std::printf("%-40s %10.4f %12.1f %9.1f%%   C %016llx\n", c.name, best, tflops,
-                100 * tflops / peak_of(c.type_in), hash);
+    std::printf("%-44s %10.4f %12.1f %9.1f%%   C %016llx\n", c.name, best, tflops,
+                100 * tflops / (c.peak > 0 ? c.peak : peak_of(c.type_in)), hash);
     std::fflush(stdout);
     CHECK(hipFree(dx));
     CHECK(hipFree(dy));

@@ -85,9 +85,13 @@ CCGLIB_API const char *ccglib_version(void);
  *                    other value: chunks of about that many bytes, whatever
  *                    the size of the job.
  *   GEMM_BLOCK_TILE  0 (default): GEMMs on tiled or whole-chunk planar
- *                    operands use 256 x 128 block tiles, or 128 x 128 ones
- *                    when the larger would leave compute units idle (small
- *                    problems); 1: always 256 x 128; 2: always 128 x 128.
+ *                    operands use 256 x 128 block tiles, 128 x 128 ones when
+ *                    the larger would leave compute units idle (small
+ *                    problems), or 192 x 256 ones (16-bit tiled input, planar C
+ *                    without alpha or beta, M and N multiples of 64, K of more
+ *                    than 32) when those fill the compute units well enough;
+ *                    1: always 256 x 128; 2: always 128 x 128; 3: 192 x 256
+ *                    wherever that kernel applies, else as 0.
  * ---------------------------------------------------------------------- */
 enum {
   CCGLIB_AMD_OPTION_INT1_POPCOUNT = 0,

@@ -456,14 +456,64 @@ def test_block_tiles_int1(block_tile, variant):
             int1_case(2, 130, 260, 1024, variant, c_axis=INTERLEAVED, seed=4)
 
 
-def test_block_tile_choice_is_invisible():
-    """The same bits whichever block tile computes them (same K order per element)."""
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.float16, VT.float16),
+                                      (VT.bfloat16, VT.float32), (VT.bfloat16, VT.bfloat16)])
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_wide_block_tile(tin, tout, c_order):
+    """GEMM_BLOCK_TILE = 3: the 192 x 256 block (16-bit tiled input, planar C without
+    alpha or beta, M and N multiples of 64, K of more than one tile) against the
+    oracle: tiles that lie inside C and tiles of which only one or two 64-column
+    groups or some of the four 64-row pieces do, two to many K tiles, more C tiles
+    than compute units, and a K with a partial last tile."""
+    with cc.option(cc.Option.gemm_block_tile, 3):
+        float_case(2, 256, 192, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=1)
+        float_case(3, 320, 448, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=2)
+        float_case(1, 64, 64, 40, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=3)
+        float_case(2, 512, 832, 1000, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=4)
+        float_case(40, 256, 576, 72, tin, tout, cc.Variant.opt, PLANAR, c_order, signed=False, seed=5)
+
+
+def test_wide_block_tile_falls_back():
+    """GEMM_BLOCK_TILE = 3 where the 192 x 256 kernel does not apply (ragged M or N,
+    alpha / beta, interleaved C, K of one tile, fp8): the other kernels compute it."""
+    with cc.option(cc.Option.gemm_block_tile, 3):
+        float_case(2, 300, 520, 96, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=1)
+        float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW,
+                   alpha=1.5 - 0.5j, beta=0.25 + 1j, seed=2)
+        float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.opt, INTERLEAVED, ROW, seed=3)
+        float_case(1, 256, 192, 32, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=4)
+        float_case(1, 256, 192, 128, VT.float8e4m3, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=5)
+        float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.basic, PLANAR, ROW, seed=6)
+
+
+@pytest.mark.parametrize("B,M,N,K", [(2, 384, 640, 256), (3, 512, 4096, 576), (1, 1024, 1216, 2048)])
+def test_block_tile_choice_is_invisible(B, M, N, K):
+    """The same bits whichever block tile computes them (same K order per element, and
+    per K tile the same order of the four real products)."""
     rng = np.random.default_rng(11)
-    B, M, N, K = 2, 384, 640, 256
+    qa = quantize(rng.standard_normal((B, 2, M, K)).astype(np.float32), VT.float16).reshape(-1)
+    qb = quantize(rng.standard_normal((B, 2, N, K)).astype(np.float32), VT.float16).reshape(-1)
+    results = []
+    for block_tile in (0, 1, 2, 3):
+        with cc.option(cc.Option.gemm_block_tile, block_tile):
+            results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt))
+    for r in results[1:]:
+        assert np.array_equal(results[0], r)
+
+
+def test_wide_block_more_than_64_tiles_per_block():
+    """A block of the 192 x 256 kernel looks the coordinates of its first 64 C tiles up in a
+    table and works out the others one by one: 20000 one-tile batches are more than 64 tiles
+    for each of the 256 persistent blocks. Same bits as the 256 x 128 kernel."""
+    rng = np.random.default_rng(12)
+    B, M, N, K = 20000, 64, 64, 64
     qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), VT.float16).reshape(-1)
     qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), VT.float16).reshape(-1)
     results = []
-    for block_tile in (0, 1, 2):
+    for block_tile in (1, 3):
         with cc.option(cc.Option.gemm_block_tile, block_tile):
             results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt))
-    assert np.array_equal(results[0], results[1]) and np.array_equal(results[1], results[2])
+    assert np.array_equal(results[0], results[1])
+    want = orc.gemm(qa[:4 * 2 * M * K], qb[:4 * 2 * N * K], M, N, K, ORC_TYPE[VT.float16],
+                    ORC_TYPE[VT.float32])
+    assert np.allclose(results[1][:4], want.reshape(4, 2, M, N), rtol=1e-3, atol=1e-3)
