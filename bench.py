@@ -126,7 +126,8 @@ def check_result(name, a, b, c, torch):
             "batch": bi}
 
 
-def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_calibration=False):
+def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_calibration=False,
+            check=True):
     """Builds the step of a workload, settles, times `steps` steps and checks the result.
     Returns a dict of figures plus what the optional extra measurements need."""
     stream = torch.cuda.current_stream().cuda_stream
@@ -162,13 +163,14 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
     b_t = torch.empty(B * 2 * np_ * kp * bits // 8, dtype=torch.uint8, device="cuda")
     tr_a = cc.Transpose(B, M, K, mb, kc, bits, 0, stream, axis)
     tr_b = cc.Transpose(B, N, K, nb, kc, bits, 0, stream, axis)
-    # both operands in one launch (what Pipeline.Run does too); each on its own is
+    # both operands through one call (what Pipeline.Run does too); each on its own is
     # timed after the steps, see `standalone` below
     bytes_a, bytes_b = 2.0 * B * 2 * M * K * bits / 8, 2.0 * B * 2 * N * K * bits / 8
     kernels.append(("transposes", lambda sa=a_cur, sb=b_cur: cc.Transpose.RunPair(
         tr_a, sa.data_ptr(), a_t.data_ptr(), tr_b, sb.data_ptr(), b_t.data_ptr()), bytes_a + bytes_b))
     standalone = [("transpose_a", lambda s=a_cur: tr_a.Run(s.data_ptr(), a_t.data_ptr()), bytes_a),
-                  ("transpose_b", lambda s=b_cur: tr_b.Run(s.data_ptr(), b_t.data_ptr()), bytes_b)]
+                  ("transpose_b", lambda s=b_cur: tr_b.Run(s.data_ptr(), b_t.data_ptr()), bytes_b),
+                  ("transposes_back_to_back", kernels[-1][1], bytes_a + bytes_b)]
     gemm = cc.GEMM(B, M, N, K, 0, stream, prec, cc.Variant.opt, AX.complex_planar, MO.row_major)
     run_gemm = lambda: gemm.Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
 
@@ -247,24 +249,27 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
         per_kernel[label + "_ms"] = ms
         per_kernel[label + "_gbs"] = nbytes / ms / 1e6
         per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
-    per_kernel["method"] = ("gemm, transposes (both operands, one launch) and packing_*: event pairs "
-                            "inside the timed steps; transpose_a / transpose_b: separate launches, "
-                            "20 back to back between two events after the steps")
+    per_kernel["method"] = ("gemm, transposes (both operands through ccglib_transpose_run_pair: one "
+                            "launch when one operand is small, else two) and packing_*: event pairs "
+                            "inside the timed steps; transpose_a / transpose_b / "
+                            "transposes_back_to_back (the pair call again): 20 back to back between "
+                            "two events after the steps")
 
+    # (the library says which of its kernels the GEMM object launches)
+    kernel_name = "%s <%s -> %s>" % (gemm.KernelName(), tin_name, tout_name)
     if tin == VT.int1:
         dtype, peak, unit = "fp4 (+-1, exact int32 result)", FP4_PEAK_TOPS, "TOP/s"
-        kernel_name = "complex_gemm_mfma_dtl<int1->int32> (fp4 MFMA, bits expanded in registers)"
+        kernel_name += " (fp4 MFMA, bits expanded in registers)"
     else:
         dtype = {"float16": "f16", "bfloat16": "bf16"}.get(tin_name, "fp8")
         peak, unit = MFMA_PEAK_TFLOPS[dtype], "TFLOP/s"
-        kernel_name = "complex_gemm_mfma_dtl<%s->%s>" % (tin_name, tout_name)
 
     out = {"name": name, "description": description, "shape": (B, M, N, K), "flops": flops,
            "ms_per_step": ms_per_step, "value": flops / (ms_per_step * 1e-3) / 1e12,
            "gemm_ms": gemm_ms, "gemm_tflops": gemm_tflops, "per_kernel": per_kernel,
            "dtype": dtype, "peak": peak, "unit": unit, "kernel_name": kernel_name,
            "settle_ms": settled, "settle_steps": settle_steps, "info": info,
-           "check": check_result(name, a_in, b_in, c, torch)}
+           "check": check_result(name, a_in, b_in, c, torch) if check else None}
     if isolated:
         # the GEMM launched back to back on its own (inputs and caches warm)
         iters = max(steps, 10)
@@ -324,7 +329,8 @@ def main():
     B, M, N, K, tin_name, tout_name, axis_name, description = WORKLOADS[name]
     tin, tout = VT[tin_name], VT[tout_name]
     m = measure(name, args.steps, args.warmup, args.settle_ms, torch, np, cc,
-                isolated=args.isolated, copy_calibration=args.copy_calibration)
+                isolated=args.isolated, copy_calibration=args.copy_calibration,
+                check=not args.no_check)
     a_in, b_in, c = m.pop("_buffers")
     flops, value, ms_per_step = m["flops"], m["value"], m["ms_per_step"]
     gemm_ms, gemm_tflops, peak = m["gemm_ms"], m["gemm_tflops"], m["peak"]
@@ -434,8 +440,9 @@ def main():
         del a_in, b_in, c, m
         torch.cuda.empty_cache()
         others = {}
-        for other in ("square_bf16", "fp8_e4m3", "correlator_int1"):
-            o = measure(other, args.other_steps, 3, args.settle_ms, torch, np, cc)
+        for other in ("square_bf16", "square_bf16_out", "fp8_e4m3", "fp8_e5m2", "correlator_int1"):
+            o = measure(other, args.other_steps, 3, args.settle_ms, torch, np, cc,
+                        check=not args.no_check)
             o.pop("_buffers")
             others[other] = {
                 "kernel": o["kernel_name"], "shape": dict(zip("BMNK", o["shape"])),

@@ -93,6 +93,7 @@ class Option(enum.IntEnum):
     basic_retile = 1
     host_chunk_bytes = 2
     gemm_block_tile = 3
+    expect_unaligned = 4
 
 
 def set_option(option, value):
@@ -155,6 +156,13 @@ class GEMM(_Handle):
 
     def Run(self, d_a, d_b, d_c):
         _capi.check(_capi.load().ccglib_gemm_run(self._h, _ptr(d_a), _ptr(d_b), _ptr(d_c)))
+
+    def KernelName(self):
+        """Which kernel Run launches for 16-byte aligned buffers (no counterpart in
+        the reference)."""
+        buf = ctypes.create_string_buffer(160)
+        _capi.check(_capi.load().ccglib_gemm_kernel_name(self._h, buf, len(buf)))
+        return buf.value.decode()
 
     @staticmethod
     def GetDimensions(precision, variant=Variant.opt):

@@ -19,6 +19,7 @@ SIGNATURES = {
     "ccglib_gemm_create": (_i, [_pvp, _sz, _sz, _sz, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _i,
                                 _f, _f, _f, _f]),
     "ccglib_gemm_run": (_i, [_vp, _vp, _vp, _vp]),
+    "ccglib_gemm_kernel_name": (_i, [_vp, ctypes.c_char_p, _sz]),
     "ccglib_gemm_destroy": (_i, [_vp]),
     "ccglib_gemm_get_dimensions": (_i, [_i, _i, _i, _pu, _pu, _pu]),
     "ccglib_transpose_create": (_i, [_pvp, _sz, _sz, _sz, _sz, _sz, _sz, _i, _vp, _i]),

@@ -178,7 +178,7 @@ struct ccglib_pipeline {
 namespace {
 
 // Process-wide options (ccglib_amd_set_option), read when an object is created.
-size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0, 0};
+size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0, 0, 0};
 
 // Largest buffer of 1-bit tiles a pipeline allocates; beyond it the pipeline
 // runs the reference's sequence of kernels on its packed / transposed buffers.
@@ -209,6 +209,17 @@ void make_retile_workspace(ccglib_gemm *g) {
     g->workspace = nullptr;
     (void)hipGetLastError();
   }
+}
+
+// Whether work submitted to the stream is being recorded into a graph: nothing
+// may be allocated then (an allocation would invalidate the capture).
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
 }
 
 // Launch parameters of a GEMM object for the given buffers.
@@ -387,7 +398,8 @@ int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M, size_t N, size_t
   // times faster than the ones that load ragged rows through registers.
   // (Operands that are not 16-byte aligned get the same workspace at their first Run.)
   const size_t row_bytes = type_in == kInt1 ? ceil_div(K, 32) * 4 : K * (size_t)bits_of(type_in) / 8;
-  if (variant == kBasic && B && M && N && K && row_bytes % 16 != 0 &&
+  if (variant == kBasic && B && M && N && K &&
+      (row_bytes % 16 != 0 || g_options[CCGLIB_AMD_OPTION_EXPECT_UNALIGNED] != 0) &&
       (type_in != kInt1 || g->int1_direct)) {
     make_retile_workspace(g);
   }
@@ -423,8 +435,11 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
     const bool misaligned = (uintptr_t)d_a % 16 != 0 || (uintptr_t)d_b % 16 != 0;
     // Planar operands that are not 16-byte aligned cannot be copied to LDS in
     // place either: the object gets its workspace at the first such Run (the one
-    // allocation a Run may make) and keeps it.
-    if (misaligned && !g->retile) make_retile_workspace(g);
+    // allocation a Run may make) and keeps it - unless the stream is being
+    // captured into a graph, where the kernel that reads such rows through
+    // registers runs instead (the option EXPECT_UNALIGNED makes the object
+    // allocate at construction).
+    if (misaligned && !g->retile && !stream_is_capturing(g->stream)) make_retile_workspace(g);
     retile_now = g->retile && (misaligned || row_bytes % 16 != 0);
   }
   if (retile_now) {
@@ -455,6 +470,26 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
   const hipError_t e = (g->type_in == kInt1) ? launch_gemm_int1(p, g->stream)
                                               : launch_gemm_mfma(p, g->stream);
   if (e != hipSuccess) return fail_hip(e, "GEMM kernel launch");
+  return CCGLIB_OK;
+}
+
+int ccglib_gemm_kernel_name(ccglib_gemm_t g, char *name, size_t size) {
+  if (!g || !name || size == 0) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null argument");
+  // 16-byte aligned buffers assumed (what Run meets with memory from hipMalloc)
+  GemmParams p;
+  fill_gemm_params(g, nullptr, nullptr, nullptr, &p);
+  const char *what;
+  if (g->type_in == kInt1 && !g->int1_direct) {
+    what = "complex_gemm_int1, 128x128 block, XOR + population count";
+  } else if (g->retile) {
+    p.variant = kOpt;
+    what = describe_gemm_mfma(p);
+  } else if (g->type_in == kInt1 && g->variant == kBasic && (ceil_div(g->K, 32) * 4) % 16 != 0) {
+    what = "complex_gemm_int1, 128x128 block, XOR + population count";
+  } else {
+    what = describe_gemm_mfma(p);
+  }
+  std::snprintf(name, size, "%s%s", g->retile ? "transpose_vec (re-tiling) + " : "", what);
   return CCGLIB_OK;
 }
 
@@ -889,6 +924,15 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
                             beta_im);  // :102-105
     if (rc == CCGLIB_OK) p->gemm->input_interleaved = fused;
     p->fused = fused || planar_in_place;   // (both need 16-byte aligned rows at Run)
+    if (rc == CCGLIB_OK && p->fused && allow_fused &&
+        g_options[CCGLIB_AMD_OPTION_EXPECT_UNALIGNED] != 0) {
+      // the pipeline with transposes that takes over for unaligned buffers, now
+      // rather than at the first Run that meets them
+      rc = pipeline_create(&p->unfused, B, M, N, K, device, stream, input_complex_axis_location,
+                           output_complex_axis_location, a_mem_order, b_mem_order, c_mem_order,
+                           input_type, output_type, variant, alpha_re, alpha_im, beta_re, beta_im,
+                           false);
+    }
   } while (false);
   if (rc != CCGLIB_OK) {
     const std::string keep = g_last_error;
@@ -924,6 +968,12 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
     // element-aligned address. The pipeline that runs them is created here, once
     // (the one allocation a device Run may make), and kept.
     if (!p->unfused) {
+      if (stream_is_capturing(p->stream)) {
+        return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
+                    "pipeline input is not 16-byte aligned: the pipeline with transposes that takes "
+                    "such buffers cannot be allocated while the stream is being captured (run once "
+                    "before the capture, or create the pipeline with the option EXPECT_UNALIGNED)");
+      }
       rc = pipeline_create(&p->unfused, p->B, p->M, p->N, p->K, p->device, p->stream, p->in_axis,
                            p->c_axis, p->a_order, p->b_order, p->c_order, p->type_in, p->type_out,
                            p->variant, p->alpha_re, p->alpha_im, p->beta_re, p->beta_im, false);

@@ -98,6 +98,7 @@ bool gemm_int1_can_take_bytes(const GemmParams &p);
 hipError_t launch_gemm_int1_from_bytes(const GemmParams &p, hipStream_t stream);
 
 hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream);
+const char *describe_gemm_mfma(const GemmParams &p);
 hipError_t launch_gemm_int1(const GemmParams &p, hipStream_t stream);
 
 struct TransposeParams {

@@ -2182,6 +2182,34 @@ hipError_t launch_gemm_mfma_int1(const GemmParams &p, hipStream_t stream) {
 #endif
 
 #if CCGLIB_GEMM_MFMA_HAS(0)
+// Which kernel launch_gemm_mfma starts for these parameters (the decisions of
+// launch_typed, in words).
+const char *describe_gemm_mfma(const GemmParams &p) {
+  const bool bits8 = p.type_in == kFloat8e4m3 || p.type_in == kFloat8e5m2;
+  const bool bits16 = p.type_in == kFloat16 || p.type_in == kBfloat16;
+  const bool int1 = p.type_in == kInt1;
+  const size_t k_bytes = (size_t)p.k * bits_of(p.type_in) / 8;
+  const bool planar_direct = (p.variant == kBasic) && (k_bytes >= 16) && (k_bytes % 16 == 0) &&
+                             ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.y % 16 == 0);
+  const double penalty = int1 ? 1.0 : bits8 ? 1.05 : 1.15;
+  if (p.input_interleaved) {
+    return small_tiles_pay(p, penalty) ? "complex_gemm_mfma_dtl, 128x128 block, interleaved rows"
+                                       : "complex_gemm_mfma_dtl, 256x128 block, interleaved rows";
+  }
+  if (p.variant == kOpt || planar_direct || int1) {
+    if (bits16 && wide_tiles_apply(p) && wide_tiles_pay(p)) {
+      return "complex_gemm_mfma_wide, 192x256 block, one wave per SIMD";
+    }
+    if (p.variant == kOpt) {
+      return small_tiles_pay(p, penalty) ? "complex_gemm_mfma_dtl, 128x128 block, tiled operands"
+                                         : "complex_gemm_mfma_dtl, 256x128 block, tiled operands";
+    }
+    return small_tiles_pay(p, penalty) ? "complex_gemm_mfma_dtl, 128x128 block, planar rows"
+                                       : "complex_gemm_mfma_dtl, 256x128 block, planar rows";
+  }
+  return "complex_gemm_mfma, 128x128 block, planar rows through registers";
+}
+
 hipError_t launch_gemm_mfma(const GemmParams &p, hipStream_t stream) {
   switch (p.type_in) {
     case kFloat16: return launch_gemm_mfma_f16(p, stream);

@@ -92,13 +92,23 @@ CCGLIB_API const char *ccglib_version(void);
  *                    than 32) when those fill the compute units well enough;
  *                    1: always 256 x 128; 2: always 128 x 128; 3: 192 x 256
  *                    wherever that kernel applies, else as 0.
+ *   EXPECT_UNALIGNED 0 (default): a basic-variant GEMM that meets operands that
+ *                    are not 16-byte aligned allocates its tiled copies at that
+ *                    Run, and a pipeline that reads rows in place creates the
+ *                    pipeline with transposes that takes over for such buffers
+ *                    at that Run (never while the stream is being captured
+ *                    into a graph: the GEMM then reads the rows through
+ *                    registers, the pipeline reports an error); 1: both are
+ *                    allocated when the object is created, and no device Run
+ *                    allocates.
  * ---------------------------------------------------------------------- */
 enum {
   CCGLIB_AMD_OPTION_INT1_POPCOUNT = 0,
   CCGLIB_AMD_OPTION_BASIC_RETILE = 1,
   CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES = 2,
   CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE = 3,
-  CCGLIB_AMD_OPTION_COUNT = 4
+  CCGLIB_AMD_OPTION_EXPECT_UNALIGNED = 4,
+  CCGLIB_AMD_OPTION_COUNT = 5
 };
 CCGLIB_API int ccglib_amd_set_option(int option, size_t value);
 CCGLIB_API int ccglib_amd_get_option(int option, size_t *value);
@@ -144,6 +154,11 @@ CCGLIB_API int ccglib_gemm_create(ccglib_gemm_t *gemm, size_t B, size_t M,
 /* Argument order (a, b, c) as in GEMM::Run. */
 CCGLIB_API int ccglib_gemm_run(ccglib_gemm_t gemm, const void *d_a,
                                const void *d_b, void *d_c);
+/* Which kernel Run launches for 16-byte aligned buffers, in words (kernel
+ * function, block tile, operand layout). No counterpart in the reference, whose
+ * one kernel per precision is fixed by its parameter tables (src/mma/Kernel*.cpp);
+ * here the choice depends on the problem size, and benchmark output names it. */
+CCGLIB_API int ccglib_gemm_kernel_name(ccglib_gemm_t gemm, char *name, size_t size);
 CCGLIB_API int ccglib_gemm_destroy(ccglib_gemm_t gemm);
 /* (m_per_block, n_per_block, k_chunk): the chunk sizes of the opt layout. */
 CCGLIB_API int ccglib_gemm_get_dimensions(int type_in, int type_out,
@@ -174,7 +189,9 @@ CCGLIB_API int ccglib_transpose_run_host(ccglib_transpose_t transpose,
                                          const void *h_input, void *d_output);
 /* Both operands of one GEMM: the same as ccglib_transpose_run on each, in one
  * kernel launch where the two have the same batch size, row length N, N_chunk,
- * width and input layout (otherwise in two). No counterpart in the reference,
+ * width and input layout and one has at most a quarter of the other's rows
+ * (otherwise in two: operands of similar size measured 1-3 % faster one after
+ * the other). No counterpart in the reference,
  * whose pipeline launches one transpose per operand
  * (src/pipeline/Pipeline.cpp:116-121); a small operand no longer pays for a
  * launch, ramp-up and tail of its own. Both objects must have been created

@@ -115,3 +115,99 @@ def test_graph_int1(what):
         make = Steps
 
     _capture_and_replay(make, [a, b], fill, (B * 2 * M * N,), torch.int32)
+
+
+def _capture(side, run):
+    """Captures run() on the stream `side` without any Run before it; returns the graph."""
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run()
+    return graph
+
+
+@pytest.mark.parametrize("expect_unaligned", [0, 1])
+def test_graph_basic_gemm_meets_unaligned_operands_during_capture(expect_unaligned):
+    """A basic-variant GEMM allocates its re-tiling workspace at the first Run that meets
+    operands which are not 16-byte aligned - but not while the stream is being captured
+    (the allocation would invalidate the capture): there it reads the rows through
+    registers. With the option EXPECT_UNALIGNED the workspace exists from construction
+    on. Either way the first such Run can be the captured one, and the replays give the
+    oracle's result."""
+    import oracle as orc
+    from gpu_util import ORC_TYPE
+    B, M, N, K = 2, 96, 200, 72
+    rng = np.random.default_rng(31)
+    qa = quantize(rng.uniform(-1, 1, B * 2 * M * K).astype(np.float32), VT.float16)
+    qb = quantize(rng.uniform(-1, 1, B * 2 * N * K).astype(np.float32), VT.float16)
+    skew = 1   # one fp16 element: 2 bytes off a 16-byte boundary
+    d_a = to_device(np.concatenate([np.zeros(skew, np.uint16), qa]))
+    d_b = to_device(np.concatenate([np.zeros(skew, np.uint16), qb]))
+    d_c = torch.zeros(B * 2 * M * N, dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    with cc.option(cc.Option.expect_unaligned, expect_unaligned):
+        gemm = cc.GEMM(B, M, N, K, 0, side.cuda_stream, cc.Precision(VT.float16, VT.float32),
+                       cc.Variant.basic)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = _capture(side, lambda: gemm.Run(d_a.data_ptr() + 2 * skew, d_b.data_ptr() + 2 * skew,
+                                            d_c.data_ptr()))
+    assert torch.cuda.mem_get_info()[0] >= free_before, "Run allocated during the capture"
+    want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[VT.float16], ORC_TYPE[VT.float32])
+    for _ in range(2):
+        d_c.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = d_c.cpu().numpy().reshape(want.shape)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
+
+
+def test_graph_fused_pipeline_meets_unaligned_buffers_during_capture():
+    """A pipeline that reads rows in place creates the pipeline with transposes for
+    unaligned buffers at the first Run that meets them; during a capture that Run reports
+    an error instead of allocating, and with the option EXPECT_UNALIGNED the fallback
+    exists from construction on and the captured Run works."""
+    import oracle as orc
+    from gpu_util import ORC_TYPE
+    B, M, N, K = 2, 64, 128, 72
+    rng = np.random.default_rng(32)
+    a = rng.standard_normal((B, 2, M, K)).astype(np.float16)
+    b = rng.standard_normal((B, 2, N, K)).astype(np.float16)
+    skew = 2
+    il = lambda x: np.concatenate([np.zeros(skew, np.uint16),
+                                   np.ascontiguousarray(x.transpose(0, 2, 3, 1)).view(np.uint16).reshape(-1)])
+    d_a, d_b = to_device(il(a)), to_device(il(b))
+    d_c = torch.zeros(B * 2 * M * N, dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    make = lambda: cc.Pipeline(B, M, N, K, 0, side.cuda_stream, INTERLEAVED, PLANAR, ROW, COL, ROW,
+                               VT.float16, VT.float32, cc.Variant.opt)
+    run = lambda p: p.Run(d_a.data_ptr() + 2 * skew, d_b.data_ptr() + 2 * skew, d_c.data_ptr())
+    # default: the Run inside the capture refuses
+    pipe = make()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        try:
+            with pytest.raises(RuntimeError, match="cannot be allocated while the stream is being captured"):
+                run(pipe)
+        finally:
+            graph.capture_end()
+    torch.cuda.synchronize()
+    del graph
+    # with the option: captured and replayed
+    with cc.option(cc.Option.expect_unaligned, 1):
+        pipe = make()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = _capture(side, lambda: run(pipe))
+    assert torch.cuda.mem_get_info()[0] >= free_before, "Run allocated during the capture"
+    want = orc.gemm(a.view(np.uint16).reshape(-1), b.view(np.uint16).reshape(-1), M, N, K,
+                    ORC_TYPE[VT.float16], ORC_TYPE[VT.float32])
+    for _ in range(2):
+        d_c.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = d_c.cpu().numpy().reshape(want.shape)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3

@@ -84,12 +84,17 @@ def test_empty():
 
 @pytest.mark.parametrize("axis", [PLANAR, INTERLEAVED])
 @pytest.mark.parametrize("bits,kc,Ma,Mb,N,Mca,Mcb,skew", [
+    # (one launch for both when one operand has at most a quarter of the other's rows)
     (16, 32, 512, 4096, 576, 128, 128, 0),    # beamformer operands: rows of 72 vectors
-    (16, 32, 100, 300, 1000, 128, 64, 0),     # ragged rows and columns, different row tiles
-    (8, 64, 77, 130, 257, 128, 128, 0),       # rows that are not whole vectors
+    (16, 32, 70, 300, 1000, 128, 64, 0),      # ragged rows and columns, different row tiles
+    (16, 32, 100, 300, 1000, 128, 64, 0),     # the same as two launches
+    (8, 64, 30, 130, 257, 128, 128, 0),       # rows that are not whole vectors
+    (8, 64, 77, 130, 257, 128, 128, 0),
+    (32, 16, 50, 200, 96, 128, 128, 0),
     (32, 16, 64, 200, 96, 128, 128, 0),
-    (16, 32, 129, 64, 264, 128, 128, 1),      # first operand not 16-byte aligned: two launches
-    (1, 512, 100, 256, 1056, 128, 128, 0),    # 1-bit words
+    (16, 32, 129, 30, 264, 128, 128, 1),      # first operand not 16-byte aligned: two launches
+    (1, 512, 300, 64, 1056, 128, 128, 0),     # 1-bit words, the small operand second
+    (1, 512, 100, 256, 1056, 128, 128, 0),
     (16, 32, 5, 7, 7, 128, 128, 0),           # scalar kernel for both
 ])
 def test_pair_matches_oracle(axis, bits, kc, Ma, Mb, N, Mca, Mcb, skew):
