@@ -241,7 +241,10 @@ class Pipeline(_Handle):
                                                          _ptr(h_c)))
 
 
-STATIC_SCRATCH_BYTES = 32 << 20   # CCGLIB_AMD_STATIC_SCRATCH_BYTES in include/ccglib_amd.h
+def static_scratch_bytes():
+    """Size of the static device array behind pipeline_run_static in the loaded library
+    (build option CCGLIB_AMD_STATIC_SCRATCH_BYTES, 32 MiB unless the build says otherwise)."""
+    return _capi.load().ccglib_amd_static_scratch_bytes()
 
 
 def pipeline_run_static(B, M, N, K, device, stream, input_complex_axis_location,

@@ -16,6 +16,7 @@ SIGNATURES = {
     "ccglib_version": (ctypes.c_char_p, []),
     "ccglib_amd_set_option": (_i, [_i, _sz]),
     "ccglib_amd_get_option": (_i, [_i, ctypes.POINTER(ctypes.c_size_t)]),
+    "ccglib_amd_static_scratch_bytes": (_sz, []),
     "ccglib_gemm_create": (_i, [_pvp, _sz, _sz, _sz, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _i,
                                 _f, _f, _f, _f]),
     "ccglib_gemm_run": (_i, [_vp, _vp, _vp, _vp]),

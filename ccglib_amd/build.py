@@ -29,6 +29,13 @@ HIPCC_FLAGS = [
 ]
 
 
+def _defines():
+    """Build options taken from the environment: CCGLIB_AMD_STATIC_SCRATCH_BYTES, the size
+    of the static device array of ccglib_pipeline_run_static (default in the header)."""
+    v = os.environ.get("CCGLIB_AMD_STATIC_SCRATCH_BYTES")
+    return ["-DCCGLIB_AMD_STATIC_SCRATCH_BYTES=((size_t)%d)" % int(v)] if v else []
+
+
 def _hipcc():
     return shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
@@ -45,7 +52,7 @@ def _compile(src, force):
     path = os.path.join(CSRC, src)
     if not force and not _stale(obj, [path] + HEADERS):
         return obj, ""
-    cmd = [_hipcc()] + HIPCC_FLAGS + ["-c", path, "-o", obj]
+    cmd = [_hipcc()] + HIPCC_FLAGS + _defines() + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
                     if "packed-fp32-ops" not in l)

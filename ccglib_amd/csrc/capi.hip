@@ -1166,6 +1166,8 @@ namespace {
 // memory it allocates. One array per GPU, held from the moment the library's
 // code is loaded there until the process ends; every call on that GPU uses it.
 constexpr size_t kStaticScratchBytes = CCGLIB_AMD_STATIC_SCRATCH_BYTES;
+static_assert(kStaticScratchBytes >= 256 && kStaticScratchBytes % 256 == 0,
+              "CCGLIB_AMD_STATIC_SCRATCH_BYTES must be a positive multiple of 256");
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Device address of `scratch` on each GPU. In host code the array's name is only
@@ -1197,6 +1199,8 @@ size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
 }  // namespace
 
 extern "C" {
+
+size_t ccglib_amd_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int ccglib_pipeline_run_static(size_t B, size_t M, size_t N, size_t K, int device, void *stream,
                                int input_complex_axis_location,

@@ -20,6 +20,14 @@
 //   exponents; fp8 without sign bit), kept for comparison with their files.
 // --fill=zero: all-zero operands (no power limit).
 // `make ABLATE=n` builds timing-only variants (see CCGLIB_ABLATE in gemm_mfma.hip).
+//
+//   ./tune_gemm --probe=mfma|mix|fill|l2read [--fill=...]
+// Small probes of the machine that the kernels' floors are argued from: the rate
+// of matrix instructions issued from registers alone (1 or 2 waves per SIMD, the
+// operands changing from instruction to instruction), what an instruction between
+// two matrix instructions costs a wave that has the SIMD to itself, the rate of a
+// plain fill of 1 GiB, and the rate at which all compute units read a window of a
+// given size over and over (L2 and memory-side cache).
 #include "../csrc/gemm_mfma.hip"
 #include "../csrc/gemm_int1.hip"
 
@@ -209,13 +217,203 @@ static void fill_legacy(void *d, size_t bytes, int type) {
     CHECK(hipMemcpy((char *)d + o, h.data(), std::min(h.size() * 2, bytes - o), hipMemcpyHostToDevice));
 }
 
+
+// ---- probes ------------------------------------------------------------------------
+typedef float f16v_t __attribute__((ext_vector_type(16)));
+
+// MFMAs from registers only. SHAPE 16: 16x16x32, 32: 32x32x16 (fp16). Four A and
+// four B operand sets take turns so that the inputs change as in a GEMM.
+template <int SHAPE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES / 4) void probe_mfma(const int4_t *in, float *out, int iters) {
+  extern __shared__ char probe_lds[];
+  int4_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = in[(threadIdx.x % 64) * 8 + i];
+    b[i] = in[(threadIdx.x % 64) * 8 + 4 + i];
+  }
+  constexpr int NACC = SHAPE == 16 ? 16 : 8;
+  typename AccType<SHAPE>::type acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 64; ++n) {
+      if constexpr (SHAPE == 16) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[n % NACC]) : "v"(a[n % 4]), "v"(b[(n / 4) % 4]));
+      } else {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[n % NACC]) : "v"(a[n % 4]), "v"(b[(n / 4) % 4]));
+      }
+    }
+  }
+  asm volatile("s_nop 15\n\ts_nop 15");
+  float s = 0;
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) s += acc[i][0] + acc[i][3];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// What an instruction between two 16x16x32 MFMAs costs one wave per SIMD. MODE 0:
+// none; 1 / 2: one / two vector-ALU instructions behind every MFMA; 3: four in a row
+// behind every fourth; 4: a ds_read_b128 behind every eighth; 5: a 1 KiB global ->
+// LDS copy behind every twelfth; 6: four such copies in a row behind every 48th.
+template <int MODE>
+__global__ __launch_bounds__(256, 1) void probe_mix(const int4_t *in, float *out, int iters) {
+  extern __shared__ __attribute__((aligned(1024))) char probe_lds[];
+  int4_t a = in[(threadIdx.x % 64) * 8], b = in[(threadIdx.x % 64) * 8 + 4];
+  float4_t acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  int x0 = a[0], x1 = a[1], x2 = a[2], x3 = a[3];
+  int4_t l = {0, 0, 0, 0};
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)probe_lds;
+  const unsigned la = lds_base + 65536 + (threadIdx.x % 64) * 16;
+  const unsigned wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / 64));
+  const char *src = reinterpret_cast<const char *>(in);
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 96; ++n) {
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[n % 16]) : "v"(a), "v"(b));
+      if (MODE == 1 || MODE == 2) asm volatile("v_xor_b32 %0, 0x80008000, %0" : "+v"(x0));
+      if (MODE == 2) asm volatile("v_xor_b32 %0, 0x80008000, %0" : "+v"(x1));
+      if (MODE == 3 && (n & 3) == 3) {
+        asm volatile("v_xor_b32 %0, 0x80008000, %0\n\tv_xor_b32 %1, 0x80008000, %1\n\t"
+                     "v_xor_b32 %2, 0x80008000, %2\n\tv_xor_b32 %3, 0x80008000, %3"
+                     : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
+      }
+      if (MODE == 4 && (n & 7) == 7) asm volatile("ds_read_b128 %0, %1" : "=v"(l) : "v"(la));
+      if (MODE == 5 && n % 12 == 11) load_1k_to_lds(src, (threadIdx.x % 64) * 16, lds_base + wave * 8192 + (n / 12) * 1024);
+      if (MODE == 6 && n % 48 == 47) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) load_1k_to_lds(src, (threadIdx.x % 64) * 16, lds_base + wave * 8192 + c * 1024);
+      }
+    }
+    if (MODE == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(l));
+    if (MODE == 5 || MODE == 6) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  asm volatile("s_nop 15\n\ts_nop 15");
+  float s = x0 + x1 + x2 + x3 + l[0];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i][0];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ void probe_fill(float4_t *out, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    out[i] = float4_t{1.f, 2.f, 3.f, 4.f};
+  }
+}
+// every block reads the whole window `rounds` times, each block starting elsewhere
+__global__ void probe_window_read(const int4_t *in, size_t n, int rounds, int *sink) {
+  int4_t s = {0, 0, 0, 0};
+  const size_t start = (blockIdx.x * 977u % 1024u) * (n / 1024);
+  for (int r = 0; r < rounds; ++r) {
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
+      size_t j = i + start;
+      j = j >= n ? j - n : j;
+      const int4_t v = in[j];
+      s[0] ^= v[0];
+      s[1] ^= v[1];
+      s[2] ^= v[2];
+      s[3] ^= v[3];
+    }
+  }
+  if ((s[0] ^ s[1] ^ s[2] ^ s[3]) == 0x12345678) *sink = 1;
+}
+
+template <typename F> static float time_launches(F &&launch, int reps) {
+  hipEvent_t e0, e1;
+  CHECK(hipEventCreate(&e0));
+  CHECK(hipEventCreate(&e1));
+  float ms = 0;
+  for (int round = 0; round < 2; ++round) {   // the second round is the settled one
+    CHECK(hipEventRecord(e0));
+    for (int i = 0; i < reps; ++i) launch();
+    CHECK(hipEventRecord(e1));
+    CHECK(hipEventSynchronize(e1));
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+  }
+  return ms / reps;
+}
+
+static int run_probe(const std::string &probe, const std::string &fill) {
+  int4_t *in;
+  float *out;
+  CHECK(hipMalloc(&in, 1 << 20));
+  CHECK(hipMalloc(&out, 256 * 512 * 4));
+  if (fill == "zero") {
+    CHECK(hipMemset(in, 0, 1 << 20));
+  } else {
+    fill_baseline(in, 1 << 20, kFloat16, kLoadInterleavedVec, 1, false, 7);
+  }
+  CHECK(hipDeviceSynchronize());
+  const int iters = 4000;
+  if (probe == "mfma") {
+    std::printf("matrix instructions from registers only, %s operands (four A and four B sets in turn), fp16\n", fill.c_str());
+    auto run = [&](const char *name, auto kernel, int waves, double flop_per_mfma) {
+      CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024));
+      const float ms = time_launches([&] { hipLaunchKernelGGL(kernel, dim3(256), dim3(64 * waves), 100 * 1024, 0, in, out, iters); }, 10);
+      const double tflops = 64.0 * flop_per_mfma * iters * waves * 256 / (ms * 1e-3) / 1e12;
+      std::printf("%-32s %8.3f ms %8.1f TFLOP/s  %5.1f%% of 2516.6\n", name, ms, tflops, 100 * tflops / 2516.6);
+    };
+    run("16x16x32, 1 wave per SIMD", probe_mfma<16, 4>, 4, 2.0 * 16 * 16 * 32);
+    run("16x16x32, 2 waves per SIMD", probe_mfma<16, 8>, 8, 2.0 * 16 * 16 * 32);
+    run("32x32x16, 1 wave per SIMD", probe_mfma<32, 4>, 4, 2.0 * 32 * 32 * 16);
+    run("32x32x16, 2 waves per SIMD", probe_mfma<32, 8>, 8, 2.0 * 32 * 32 * 16);
+  } else if (probe == "mix") {
+    std::printf("one wave per SIMD issuing 16x16x32 MFMAs and, between them (%s operands):\n", fill.c_str());
+    auto run = [&](const char *name, auto kernel) {
+      CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024));
+      const float ms = time_launches([&] { hipLaunchKernelGGL(kernel, dim3(256), dim3(256), 100 * 1024, 0, in, out, iters); }, 10);
+      const double tflops = 96.0 * 2 * 16 * 16 * 32 * iters * 4 * 256 / (ms * 1e-3) / 1e12;
+      std::printf("%-52s %8.3f ms %8.1f TFLOP/s  %5.1f%% of 2516.6\n", name, ms, tflops, 100 * tflops / 2516.6);
+    };
+    run("nothing", probe_mix<0>);
+    run("one v_xor behind every MFMA", probe_mix<1>);
+    run("two v_xor behind every MFMA", probe_mix<2>);
+    run("four v_xor in a row behind every 4th MFMA", probe_mix<3>);
+    run("a ds_read_b128 behind every 8th MFMA", probe_mix<4>);
+    run("a 1 KiB global -> LDS copy behind every 12th MFMA", probe_mix<5>);
+    run("four such copies in a row behind every 48th MFMA", probe_mix<6>);
+  } else if (probe == "fill") {
+    for (size_t mib : {16, 256, 1024}) {
+      float4_t *buf;
+      CHECK(hipMalloc(&buf, mib << 20));
+      const size_t n = (mib << 20) / 16;
+      const float ms = time_launches([&] { hipLaunchKernelGGL(probe_fill, dim3(8192), dim3(256), 0, 0, buf, n); }, 20);
+      std::printf("fill of %5zu MiB: %8.4f ms  %6.2f TB/s\n", mib, ms, (double)(mib << 20) / (ms * 1e-3) / 1e12);
+      CHECK(hipFree(buf));
+    }
+  } else if (probe == "l2read") {
+    int *sink;
+    CHECK(hipMalloc(&sink, 4));
+    for (size_t kib : {1024, 2048, 4096, 16384, 65536, 262144}) {
+      int4_t *buf;
+      CHECK(hipMalloc(&buf, kib << 10));
+      CHECK(hipMemset(buf, 1, kib << 10));
+      const size_t n = (kib << 10) / 16;
+      const int rounds = (int)std::max<size_t>(1, (64 << 10) / kib);
+      const float ms = time_launches([&] { hipLaunchKernelGGL(probe_window_read, dim3(1024), dim3(256), 0, 0, buf, n, rounds, sink); }, 5);
+      std::printf("1024 blocks reading a window of %7zu KiB: %8.4f ms  %6.2f TB/s\n", kib, ms,
+                  1024.0 * rounds * (kib << 10) / (ms * 1e-3) / 1e12);
+      CHECK(hipFree(buf));
+    }
+  } else {
+    std::printf("unknown probe '%s' (mfma, mix, fill or l2read)\n", probe.c_str());
+    return 1;
+  }
+  return 0;
+}
+
 int main(int argc, char **argv) {
   unsigned B = 64, M = 512, N = 4096, K = 576;
-  std::string fill = std::getenv("ZERO") ? "zero" : "baseline";
+  std::string fill = std::getenv("ZERO") ? "zero" : "baseline", probe;
   std::vector<const char *> pos;
   for (int i = 1; i < argc; ++i) {
     if (std::strncmp(argv[i], "--fill=", 7) == 0) {
       fill = argv[i] + 7;
+    } else if (std::strncmp(argv[i], "--probe=", 8) == 0) {
+      probe = argv[i] + 8;
     } else {
       pos.push_back(argv[i]);
     }
@@ -224,6 +422,7 @@ int main(int argc, char **argv) {
     std::printf("unknown fill '%s' (baseline, legacy or zero)\n", fill.c_str());
     return 1;
   }
+  if (!probe.empty()) return run_probe(probe, fill);
   if (pos.size() >= 4) {
     B = (unsigned)std::atoi(pos[0]);
     M = (unsigned)std::atoi(pos[1]);

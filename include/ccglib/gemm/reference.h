@@ -42,12 +42,26 @@ inline void from_float(float v, float *out) { *out = v; }
 inline void from_float(float v, half *out) { *out = __float2half(v); }
 inline void from_float(float v, bf16 *out) { *out = __float2bfloat16(v); }
 
+// A float product that is rounded before anything is added to it, whatever the
+// compiler and its flags (-mfma with -ffp-contract=fast fuses across statements
+// and, in clang, past `#pragma clang fp contract(off)` too): the value passes
+// through an empty asm statement, which no optimiser looks into, so there is no
+// multiply left next to an add that could become a fused multiply-add.
+inline float rounded_product(float x, float y) {
+  float p = x * y;
+#if defined(__x86_64__)
+  __asm__ volatile("" : "+x"(p));
+#elif defined(__aarch64__)
+  __asm__ volatile("" : "+w"(p));
+#else
+  __asm__ volatile("" : "+m"(p));
+#endif
+  return p;
+}
+
 template <typename Tin, typename Tout>
 void gemm_float(const Tin *a, const Tin *b, Tout *c, size_t M, size_t N, size_t K,
                 ccglib::mma::MemOrder order, std::complex<float> alpha, std::complex<float> beta) {
-#if defined(__clang__)
-#pragma clang fp contract(off)  // every product and sum rounded on its own, whatever the build flags
-#endif
   const Tin *a_im = a + M * K, *b_im = b + N * K;
   Tout *c_im = c + M * N;
   const bool scale = alpha != std::complex<float>(1.f, 0.f);
@@ -58,20 +72,21 @@ void gemm_float(const Tin *a, const Tin *b, Tout *c, size_t M, size_t N, size_t 
       for (size_t k = 0; k < K; ++k) {
         const float ar = to_float(a[m * K + k]), ai = to_float(a_im[m * K + k]);
         const float br = to_float(b[n * K + k]), bi = to_float(b_im[n * K + k]);
-        const float t_re = ar * br - ai * bi, t_im = ar * bi + ai * br;
+        const float t_re = rounded_product(ar, br) - rounded_product(ai, bi);
+        const float t_im = rounded_product(ar, bi) + rounded_product(ai, br);
         re += t_re;
         im += t_im;
       }
       if (scale) {
         const float r = re;
-        re = alpha.real() * r - alpha.imag() * im;
-        im = alpha.imag() * r + alpha.real() * im;
+        re = rounded_product(alpha.real(), r) - rounded_product(alpha.imag(), im);
+        im = rounded_product(alpha.imag(), r) + rounded_product(alpha.real(), im);
       }
       const size_t at = order == ccglib::mma::row_major ? m * N + n : n * M + m;
       if (add_c) {
         const float cr = to_float(c[at]), ci = to_float(c_im[at]);
-        re += beta.real() * cr - beta.imag() * ci;
-        im += beta.imag() * cr + beta.real() * ci;
+        re += rounded_product(beta.real(), cr) - rounded_product(beta.imag(), ci);
+        im += rounded_product(beta.imag(), cr) + rounded_product(beta.real(), ci);
       }
       from_float(re, &c[at]);
       from_float(im, &c_im[at]);

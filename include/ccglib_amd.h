@@ -284,8 +284,22 @@ CCGLIB_API int ccglib_pipeline_destroy(ccglib_pipeline_t pipeline);
  *     (1-bit input: a multiple of 32).
  *   - All calls on one GPU share the array: calls whose kernels may overlap
  *     (different streams, no dependency) race. Calls on one stream are safe.
+ *   - What fits the default of 32 MiB, with M', N' the rows padded to 128 and
+ *     K' padded to the chunk: B (M' + N') K' <= 8 Mi (2^23) elements for 16-bit
+ *     input, 16 Mi for fp8, 4 Mi for float32, 128 Mi samples for 1-bit planar
+ *     input and about 64 Mi for 1-bit interleaved input (whose packed copies live
+ *     in the array too). E.g. 16-bit: B = 16 of 256 x 256 x 1024, or one
+ *     1024 x 1024 x 4096.
+ *   - The size is a build option: compile the library with
+ *     -DCCGLIB_AMD_STATIC_SCRATCH_BYTES=<bytes> (a multiple of 256;
+ *     ccglib_amd/build.py reads the environment variable of the same name).
+ *     ccglib_amd_static_scratch_bytes() returns what the loaded library was
+ *     built with, which is the figure that binds - not this header's default.
  * ---------------------------------------------------------------------- */
+#ifndef CCGLIB_AMD_STATIC_SCRATCH_BYTES
 #define CCGLIB_AMD_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+#endif
+CCGLIB_API size_t ccglib_amd_static_scratch_bytes(void);
 CCGLIB_API int ccglib_pipeline_run_static(
     size_t B, size_t M, size_t N, size_t K, int device, void *stream,
     int input_complex_axis_location, int output_complex_axis_location,

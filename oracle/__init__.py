@@ -60,6 +60,8 @@ def lib():
         L.oracle_unpack_bits.restype = None
         L.oracle_ceildiv.argtypes = [sz, sz]
         L.oracle_ceildiv.restype = sz
+        L.oracle_reference_fixture.argtypes = [vp, vp, sz, ctypes.POINTER(ctypes.c_uint)]
+        L.oracle_reference_fixture.restype = None
         for name, arg, res in [
             ("oracle_half_to_float", ctypes.c_uint16, f),
             ("oracle_bf16_to_float", ctypes.c_uint16, f),
@@ -98,19 +100,35 @@ def set_threads(n):
     lib().oracle_set_threads(n)
 
 
+def reference_fixture(n_a, n_b, words=False):
+    """The inputs of the reference's GEMM tests (test/gemm/mma.cpp:144-217): n_a values
+    for A, then n_b for B, from one libc rand_r sequence that starts at seed 0:
+    rand_r / RAND_MAX as float32 in [0, 1], or (words=True, 1-bit input) the raw 31-bit
+    values as packed words. Returns (a, b)."""
+    seed = ctypes.c_uint(0)
+    out = []
+    for n in (n_a, n_b):
+        x = np.empty(n, dtype=np.uint32 if words else np.float32)
+        lib().oracle_reference_fixture(None if words else _ptr(x), _ptr(x) if words else None, n,
+                                       ctypes.byref(seed))
+        out.append(x)
+    return out
+
+
 def gemm(a, b, M, N, K, type_in, type_out=FLOAT32, c_order=ROW_MAJOR,
-         alpha=1 + 0j, beta=0j, c_in=None):
+         alpha=1 + 0j, beta=0j, c_in=None, batch=None):
     """Batched complex GEMM C = alpha A B^T + beta C_in with the reference's CPU
     semantics; the batch loop is the caller's loop in the reference
     (test/gemm/verify.h:54-60) and lives here.
 
     a: [B][2][M][K'] b: [B][2][N][K'] (K' = K, or ceil(K/32) words for 1-bit).
     Returns c [B][2][M][N] (row major) or [B][2][N][M] (column major) in the
-    storage type of ``type_out``.
+    storage type of ``type_out``. ``batch`` is only needed where the operands are
+    empty (K = 0) and B cannot be read from their size.
     """
     alpha, beta = complex(alpha), complex(beta)
     kk = (K + 31) // 32 if type_in == INT1 else K
-    B = a.size // (2 * M * kk)
+    B = batch if batch is not None else a.size // (2 * M * kk)
     _check(a, _STORAGE[type_in], B * 2 * M * kk, "a")
     _check(b, _STORAGE[type_in], B * 2 * N * kk, "b")
     out_dt = _STORAGE[type_out]
@@ -122,8 +140,8 @@ def gemm(a, b, M, N, K, type_in, type_out=FLOAT32, c_order=ROW_MAJOR,
     else:
         _check(c_in, out_dt, B * 2 * M * N, "c_in")
         c = np.array(c_in, dtype=out_dt).reshape(shape).copy()
-    a3 = a.reshape(B, -1)
-    b3 = b.reshape(B, -1)
+    a3 = a.reshape(B, 2 * M * kk)
+    b3 = b.reshape(B, 2 * N * kk)
     L = lib()
     for i in range(B):
         ai, bi, ci = a3[i], b3[i], c[i]

@@ -31,9 +31,11 @@
  *                       library's casts (all 256 fp8 codes, all 65536 fp16 and
  *                       bf16 codes).
  */
+#define _POSIX_C_SOURCE 200809L   /* rand_r */
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* Enum values are those of the reference API
@@ -405,6 +407,22 @@ void oracle_unpack_bits(const uint32_t *in, uint8_t *out, size_t N) {
 
 /* ceildiv as in include/ccglib/common/helper.h:6-9 (positive operands). */
 size_t oracle_ceildiv(size_t a, size_t b) { return a / b + (a % b != 0); }
+
+/*
+ * The inputs of the reference's GEMM tests (test/gemm/mma.cpp:144-217): A, then
+ * B, filled element by element from ONE rand_r sequence that starts at seed 0 -
+ * rand_r / RAND_MAX in float (then converted to the input type by the caller),
+ * or the raw value for packed 1-bit words. glibc's rand_r is a fixed algorithm,
+ * so this reproduces the reference's numbers. `seed` carries the state from the
+ * call for A to the call for B. Exactly one of `values` / `words` is non-null.
+ */
+void oracle_reference_fixture(float *values, uint32_t *words, size_t n, unsigned *seed) {
+  for (size_t i = 0; i < n; ++i) {
+    const int r = rand_r(seed);
+    if (values) values[i] = (float)r / (float)RAND_MAX;
+    if (words) words[i] = (uint32_t)r;
+  }
+}
 
 /* Number of OpenMP threads the loops above will use. */
 #ifdef _OPENMP

@@ -107,3 +107,33 @@ def check_float(got, want32, want64, type_in, type_out):
         bound = max(bound, 2.0 ** -8 if type_out == cc.ValueType.bfloat16 else 2.0 ** -10)
     assert frob <= bound, f"relative Frobenius error {frob} > {bound}"
     return frob
+
+
+def capture_and_replay(make_object, inputs, fill_inputs, out_shape, out_dtype, rounds=3):
+    """make_object(stream) -> object with Run(a, b, c); inputs: list of device tensors the
+    graph reads; fill_inputs(round) writes new contents into them."""
+    side = torch.cuda.Stream()
+    obj = make_object(side.cuda_stream)
+    d_c = torch.zeros(out_shape, dtype=out_dtype, device="cuda")
+    fill_inputs(0)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):           # warm-up outside the capture
+        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+    for r in range(1, rounds + 1):
+        fill_inputs(r)
+        torch.cuda.synchronize()
+        d_c.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = d_c.clone()
+        d_c.zero_()
+        torch.cuda.synchronize()            # `side` does not wait for the stream zero_() ran on
+        with torch.cuda.stream(side):
+            obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(got, d_c), "replay %d differs from the eager run" % r
+        assert bool(d_c.ne(0).any())

@@ -167,3 +167,110 @@ def test_correlator_int1():
     want = orc.gemm(a_np.reshape(-1), b_np.reshape(-1), 16, 16, K, orc.INT1, orc.INT32,
                     c_in=np.zeros(2 * 16 * 16, np.int32))[0]
     assert np.array_equal(c[3, :, 100:116, 900:916].cpu().numpy(), want)
+
+
+def complex_c(c, batch, interleaved):
+    if interleaved:
+        return torch.complex(c[batch, ..., 0].double(), c[batch, ..., 1].double())
+    return torch.complex(c[batch, 0].double(), c[batch, 1].double())
+
+
+@pytest.mark.parametrize("c_axis", [AX.complex_planar, AX.complex_interleaved])
+def test_beamformer_fp16_alpha_beta(c_axis):
+    """The beamformer shape with beta != 0: the kernel reads the 1 GiB C it then
+    overwrites. Three batches against complex128."""
+    B, M, N, K = 64, 512, 4096, 576
+    alpha, beta = 0.5 + 0.25j, -0.75 + 0.5j
+    il = c_axis == AX.complex_interleaved
+    gen = torch.Generator(device="cuda").manual_seed(12)
+    a = torch.randn((B, 2, M, K), device="cuda", generator=gen).half()
+    b = torch.randn((B, 2, N, K), device="cuda", generator=gen).half()
+    c = torch.randn((B, M, N, 2) if il else (B, 2, M, N), device="cuda", generator=gen)
+    keep = {batch: complex_c(c, batch, il) for batch in (0, 37, 63)}
+    a_t, b_t = tiled(a, B, M, K, VT.float16), tiled(b, B, N, K, VT.float16)
+    cc.GEMM(B, M, N, K, 0, stream(), VT.float16, cc.Variant.opt, c_axis, MO.row_major, MO.row_major,
+            MO.col_major, alpha, beta).Run(a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    for batch, c_in in keep.items():
+        a64 = torch.complex(a[batch, 0].double(), a[batch, 1].double())
+        b64 = torch.complex(b[batch, 0].double(), b[batch, 1].double())
+        want = alpha * (a64 @ b64.T) + beta * c_in
+        assert float((complex_c(c, batch, il) - want).norm() / want.norm()) <= 1e-3
+
+
+def one_batch_alone(a_t, b_t, batch, B, M, N, K, vtype, c_axis):
+    """The same product for one batch by itself, from the tiles of that batch: the
+    numbers a batched launch must reproduce bit for bit wherever the batch sits."""
+    c1 = torch.empty((M, N, 2) if c_axis == AX.complex_interleaved else (2, M, N), device="cuda")
+    cc.GEMM(1, M, N, K, 0, stream(), vtype, cc.Variant.opt, c_axis).Run(
+        a_t.data_ptr() + batch * (a_t.numel() // B), b_t.data_ptr() + batch * (b_t.numel() // B),
+        c1.data_ptr())
+    torch.cuda.synchronize()
+    return c1
+
+
+def check_batches(a, b, a_t, b_t, c, B, M, N, K, vtype, c_axis, bound):
+    il = c_axis == AX.complex_interleaved
+    for batch in (0, B // 2, B - 1):
+        a64 = torch.complex(a[batch, 0].double(), a[batch, 1].double())
+        b64 = torch.complex(b[batch, 0].double(), b[batch, 1].double())
+        want = a64 @ b64.T
+        del a64, b64
+        err = float((complex_c(c, batch, il) - want).norm() / want.norm())
+        del want
+        assert err <= bound, (batch, err)
+        assert torch.equal(c[batch], one_batch_alone(a_t, b_t, batch, B, M, N, K, vtype, c_axis)), batch
+
+
+# Offsets beyond 2^32 bytes and 2^31 elements. Block tiles (option GEMM_BLOCK_TILE): 1 is
+# 256 x 128, 2 is 128 x 128, 3 is 192 x 256 (16-bit input and planar C only; elsewhere
+# it means the default choice).
+@pytest.mark.parametrize("block_tile", [1, 2, 3])
+@pytest.mark.parametrize("c_axis", [AX.complex_planar, AX.complex_interleaved])
+@pytest.mark.parametrize("vtype,tdt,bound", [(VT.float16, torch.float16, 1e-3),
+                                             (VT.float8e4m3, torch.float8_e4m3fn, 2e-2)])
+def test_c_larger_than_4_gib(vtype, tdt, bound, c_axis, block_tile):
+    B, M, N, K = 5, 16384, 16384, 64          # C: 5 x 2 GiB, 2.7e9 elements
+    cc.set_option(cc.Option.gemm_block_tile, block_tile)
+    gen = torch.Generator(device="cuda").manual_seed(13)
+    a = torch.randn((B, 2, M, K), device="cuda", generator=gen).to(tdt)
+    b = torch.randn((B, 2, N, K), device="cuda", generator=gen).to(tdt)
+    a_t, b_t = tiled(a, B, M, K, vtype), tiled(b, B, N, K, vtype)
+    il = c_axis == AX.complex_interleaved
+    c = torch.full((B, M, N, 2) if il else (B, 2, M, N), float("nan"), device="cuda")
+    assert c.numel() > 2 ** 31
+    cc.GEMM(B, M, N, K, 0, stream(), vtype, cc.Variant.opt, c_axis).Run(
+        a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    cc.set_option(cc.Option.gemm_block_tile, 0)
+    check_batches(a, b, a_t, b_t, c, B, M, N, K, vtype, c_axis, bound)
+
+
+@pytest.mark.parametrize("block_tile", [1, 2, 3])
+@pytest.mark.parametrize("c_axis", [AX.complex_planar, AX.complex_interleaved])
+@pytest.mark.parametrize("vtype,tdt,N,bound", [(VT.float16, torch.float16, 4096, 1e-3),
+                                               (VT.float8e4m3, torch.float8_e4m3fn, 8192, 2e-2)])
+def test_tiled_operand_larger_than_4_gib(vtype, tdt, N, bound, c_axis, block_tile):
+    B, M, K = 3, 128, 98304                   # the N-row operand: 4.8e9 bytes, > 2^31 elements
+    cc.set_option(cc.Option.gemm_block_tile, block_tile)
+    gen = torch.Generator(device="cuda").manual_seed(14)
+    a = torch.randn((B, 2, M, K), device="cuda", generator=gen).to(tdt)
+    b = torch.empty((B, 2, N, K), dtype=tdt, device="cuda")
+    for batch in range(B):                    # in pieces: the float32 draw is 4 x the size
+        b[batch] = torch.randn((2, N, K), device="cuda", generator=gen).to(tdt)
+    a_t, b_t = tiled(a, B, M, K, vtype), tiled(b, B, N, K, vtype)
+    assert b_t.numel() > 2 ** 32 and b.numel() > 2 ** 31
+    # the transpose itself, bit-exact, at the far end of the operand
+    kc = 64 // b.element_size()
+    want_last = b[B - 1].view(torch.uint8 if b.element_size() == 1 else torch.int16) \
+        .view(2, N // 128, 128, K // kc, kc).permute(1, 3, 0, 2, 4).contiguous().view(-1)
+    got_last = b_t.view(want_last.dtype)[(B - 1) * want_last.numel():]
+    assert torch.equal(got_last, want_last)
+    del want_last
+    il = c_axis == AX.complex_interleaved
+    c = torch.full((B, M, N, 2) if il else (B, 2, M, N), float("nan"), device="cuda")
+    cc.GEMM(B, M, N, K, 0, stream(), vtype, cc.Variant.opt, c_axis).Run(
+        a_t.data_ptr(), b_t.data_ptr(), c.data_ptr())
+    torch.cuda.synchronize()
+    cc.set_option(cc.Option.gemm_block_tile, 0)
+    check_batches(a, b, a_t, b_t, c, B, M, N, K, vtype, c_axis, bound)

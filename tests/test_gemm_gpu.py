@@ -65,8 +65,9 @@ def reference_inputs(B, M, N, K, tin, signed, seed):
     return quantize(a, tin).reshape(-1), quantize(b, tin).reshape(-1)
 
 
-def float_case(B, M, N, K, tin, tout, variant, c_axis, c_order, signed=True, alpha=1, beta=0, seed=0):
-    qa, qb = reference_inputs(B, M, N, K, tin, signed, seed)
+def float_case(B, M, N, K, tin, tout, variant, c_axis, c_order, signed=True, alpha=1, beta=0, seed=0,
+               inputs=None):
+    qa, qb = inputs if inputs is not None else reference_inputs(B, M, N, K, tin, signed, seed)
     c_in = None
     if beta != 0:
         rng = np.random.default_rng(seed + 1)
@@ -142,6 +143,20 @@ def test_basic(tin, tout, M, N, K, c_order):
 def test_opt(tin, tout, M, N, K, c_order, c_axis):
     float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=False)
     float_case(16, M, N, K, tin, tout, cc.Variant.opt, c_axis, c_order, signed=True, seed=5)
+
+
+# The reference's own test inputs, literally (test/gemm/mma.cpp:144-217): 16 batches, A
+# then B filled from one libc rand_r sequence that starts at seed 0, at the aligned and
+# the unaligned shape of test/gemm/mma.cpp:402-408, for every pair of types it tests.
+@pytest.mark.parametrize("tin,tout", FLOAT_PAIRS)
+@pytest.mark.parametrize("M,N,K", [(128, 256, 64), (100, 60, 40)])
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_reference_seeded_inputs(tin, tout, M, N, K, variant, c_order):
+    B = 16
+    a, b = orc.reference_fixture(B * 2 * M * K, B * 2 * N * K)
+    float_case(B, M, N, K, tin, tout, variant, PLANAR, c_order,
+               inputs=(quantize(a, tin), quantize(b, tin)))
 
 
 def basic_variant(variant):
@@ -254,6 +269,44 @@ def test_more_c_tiles_than_resident_blocks(tin):
     float_case(48, 256, 1024, 128, tin, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=11)
 
 
+@pytest.mark.parametrize("beta", [0, 0.5 - 0.25j])
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.bfloat16, VT.bfloat16),
+                                      (VT.float8e4m3, VT.float32), (VT.float32, VT.float32),
+                                      (VT.int1, VT.int32)])
+@pytest.mark.parametrize("c_axis", [PLANAR, INTERLEAVED])
+def test_k_zero_basic(tin, tout, beta, c_axis):
+    """An empty product: C = beta C (the basic variant; the tiled layout of the opt
+    variant has no K = 0). beta = 0 must overwrite whatever C held."""
+    B, M, N = 3, 70, 130
+    rng = np.random.default_rng(4)
+    if tout == VT.int32:
+        beta = int(beta.real * 4) if beta else 0
+        c_in = rng.integers(-1000, 1000, B * 2 * M * N).astype(np.int32)
+    else:
+        c32 = rng.uniform(-1, 1, B * 2 * M * N).astype(np.float32)
+        c_in = c32 if tout == VT.float32 else quantize(c32, tout)
+    d_c = to_device(np.ascontiguousarray(
+        c_in.reshape(B, 2, M, N).transpose(0, 2, 3, 1) if c_axis == INTERLEAVED else c_in).reshape(-1))
+    d_ab = device_zeros(64)
+    cc.GEMM(B, M, N, 0, 0, stream(), cc.Precision(tin, tout), cc.Variant.basic, c_axis, ROW, ROW, COL,
+            1, beta).Run(d_ab.data_ptr(), d_ab.data_ptr(), d_c.data_ptr())
+    torch.cuda.synchronize()
+    got = to_host(d_c, OUT_NP[tout])
+    if c_axis == INTERLEAVED:
+        got = got.reshape(B, M, N, 2).transpose(0, 3, 1, 2)
+    empty = np.zeros(0, dtype=np.uint32 if tin == VT.int1 else quantize(np.zeros(1), tin).dtype)
+    want = orc.gemm(empty, empty, M, N, 0, ORC_TYPE[tin], ORC_TYPE[tout], int(ROW), 1, beta, c_in, batch=B)
+    got = np.ascontiguousarray(got).reshape(want.shape)
+    if tout == VT.int32:
+        assert np.array_equal(got, want)
+    else:   # beta C in float; a fused multiply-add may round the last bit differently
+        gotf, wantf = dequantize(got, tout), dequantize(want, tout)
+        if beta == 0:
+            assert not gotf.any()
+        ulp = {VT.float32: 2.0 ** -23, VT.bfloat16: 2.0 ** -7}[tout]
+        assert np.abs(gotf - wantf).max() <= 2 * ulp
+
+
 def test_beta_zero_ignores_nan_in_c():
     # run_gemm poisons C with NaN whenever beta == 0: every float case above covers
     # it; this one states the property on its own
@@ -293,14 +346,17 @@ def int1_kernel(request):
     return request.param
 
 
-def int1_case(B, M, N, K, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0, seed=0):
+def int1_case(B, M, N, K, variant, c_axis=PLANAR, c_order=ROW, alpha=1, beta=0, seed=0, inputs=None):
     rng = np.random.default_rng(seed)
     kw = (K + 31) // 32
     mask = np.full(kw, 0xFFFFFFFF, dtype=np.uint32)
     if K % 32:
         mask[-1] = (1 << (K % 32)) - 1
-    a = (rng.integers(0, 2 ** 32, (B, 2, M, kw), dtype=np.uint32) & mask).reshape(-1)
-    b = (rng.integers(0, 2 ** 32, (B, 2, N, kw), dtype=np.uint32) & mask).reshape(-1)
+    if inputs is not None:
+        a, b = inputs
+    else:
+        a = (rng.integers(0, 2 ** 32, (B, 2, M, kw), dtype=np.uint32) & mask).reshape(-1)
+        b = (rng.integers(0, 2 ** 32, (B, 2, N, kw), dtype=np.uint32) & mask).reshape(-1)
     c_in = rng.integers(-2 ** 30, 2 ** 30, B * 2 * M * N).astype(np.int32)
     d_a = transpose_operand(a, B, M, K, VT.int1) if variant == cc.Variant.opt else to_device(a)
     d_b = transpose_operand(b, B, N, K, VT.int1) if variant == cc.Variant.opt else to_device(b)
@@ -344,6 +400,16 @@ def test_kat_int1(variant, int1_kernel):
                                    (256, 128, 4096)])
 def test_int1(variant, c_order, M, N, K, int1_kernel):
     int1_case(16 if M == 64 else 3, M, N, K, variant, PLANAR, c_order, seed=M)
+
+
+# the reference's 1-bit test inputs: raw rand_r values as packed words, 16 batches of
+# 64 x 64 x 256 (test/gemm/mma.cpp:204-213, 422-436)
+@pytest.mark.parametrize("variant", [cc.Variant.basic, cc.Variant.opt])
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_int1_reference_seeded_inputs(variant, c_order, int1_kernel):
+    B, M, N, K = 16, 64, 64, 256
+    inputs = orc.reference_fixture(B * 2 * M * K // 32, B * 2 * N * K // 32, words=True)
+    int1_case(B, M, N, K, variant, c_order=c_order, inputs=inputs)
 
 
 @pytest.mark.parametrize("c_order", [ROW, COL])

@@ -7,42 +7,12 @@ import pytest
 import torch
 
 import ccglib_amd as cc
-from gpu_util import quantize, to_device, transpose_operand
+from gpu_util import capture_and_replay, quantize, to_device, transpose_operand
 
 pytestmark = pytest.mark.gpu
 VT = cc.ValueType
 PLANAR, INTERLEAVED = cc.ComplexAxisLocation.complex_planar, cc.ComplexAxisLocation.complex_interleaved
 ROW, COL = cc.MemOrder.row_major, cc.MemOrder.col_major
-
-
-def _capture_and_replay(make_object, inputs, fill_inputs, out_shape, out_dtype, rounds=3):
-    """make_object(stream) -> object with Run(a, b, c); inputs: list of device tensors the
-    graph reads; fill_inputs(round) writes new contents into them."""
-    side = torch.cuda.Stream()
-    obj = make_object(side.cuda_stream)
-    d_c = torch.zeros(out_shape, dtype=out_dtype, device="cuda")
-    fill_inputs(0)
-    torch.cuda.synchronize()
-    with torch.cuda.stream(side):           # warm-up outside the capture
-        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
-    for r in range(1, rounds + 1):
-        fill_inputs(r)
-        torch.cuda.synchronize()
-        d_c.zero_()
-        graph.replay()
-        torch.cuda.synchronize()
-        got = d_c.clone()
-        d_c.zero_()
-        torch.cuda.synchronize()            # `side` does not wait for the stream zero_() ran on
-        with torch.cuda.stream(side):
-            obj.Run(inputs[0].data_ptr(), inputs[1].data_ptr(), d_c.data_ptr())
-        torch.cuda.synchronize()
-        assert torch.equal(got, d_c), "replay %d differs from the eager run" % r
-        assert bool(d_c.ne(0).any())
 
 
 def test_graph_gemm_fp16_opt():
@@ -55,7 +25,7 @@ def test_graph_gemm_fp16_opt():
         for t in (a, b):   # any bit pattern of small fp16 numbers, tile padding included
             t.copy_(torch.randint(0, 64, t.shape, generator=g, device="cuda", dtype=torch.uint8))
 
-    _capture_and_replay(lambda s: cc.GEMM(B, M, N, K, 0, s, cc.Precision(VT.float16, VT.float32),
+    capture_and_replay(lambda s: cc.GEMM(B, M, N, K, 0, s, cc.Precision(VT.float16, VT.float32),
                                           cc.Variant.opt),
                         [a, b], fill, (B * 2 * M * N,), torch.float32)
 
@@ -70,7 +40,7 @@ def test_graph_pipeline_fp16_interleaved():
         for t in (a, b):
             t.copy_(torch.randn(t.shape, generator=g, device="cuda").to(torch.float16))
 
-    _capture_and_replay(lambda s: cc.Pipeline(B, M, N, K, 0, s, INTERLEAVED, PLANAR, ROW, COL, ROW,
+    capture_and_replay(lambda s: cc.Pipeline(B, M, N, K, 0, s, INTERLEAVED, PLANAR, ROW, COL, ROW,
                                               VT.float16, VT.float32, cc.Variant.opt),
                         [a, b], fill, (B * 2 * M * N,), torch.float32)
 
@@ -114,7 +84,7 @@ def test_graph_int1(what):
                 self.gemm.Run(self.tiled[0].data_ptr(), self.tiled[1].data_ptr(), pc)
         make = Steps
 
-    _capture_and_replay(make, [a, b], fill, (B * 2 * M * N,), torch.int32)
+    capture_and_replay(make, [a, b], fill, (B * 2 * M * N,), torch.int32)
 
 
 def _capture(side, run):

@@ -68,6 +68,23 @@ def test_kat_alpha_beta_int1():
     assert c.reshape(-1).tolist() == k["c_row_major"]
 
 
+def test_reference_fixture_is_one_libc_rand_r_sequence_from_seed_zero():
+    """test/gemm/mma.cpp:144-217: A then B from one sequence. The first value of glibc's
+    rand_r at seed 0 is 1012484; the rest is checked against libc called directly."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    libc.rand_r.argtypes = [ctypes.POINTER(ctypes.c_uint)]
+    seed = ctypes.c_uint(0)
+    raw = np.array([libc.rand_r(ctypes.byref(seed)) for _ in range(300)], dtype=np.int64)
+    assert raw[0] == 1012484
+    wa, wb = orc.reference_fixture(100, 200, words=True)
+    assert np.array_equal(np.concatenate([wa, wb]), raw.astype(np.uint32))
+    fa, fb = orc.reference_fixture(100, 200)
+    want = raw.astype(np.float32) / np.float32(2 ** 31 - 1)   # RAND_MAX, converted to float
+    assert np.array_equal(np.concatenate([fa, fb]), want)
+    assert fa.min() >= 0 and fb.max() <= 1
+
+
 def test_ceildiv():
     for a, b, want in KATS["ceildiv"]["cases"]:
         assert orc.ceildiv(a, b) == want

@@ -16,12 +16,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 KATS = json.load(open(os.path.join(HERE, "golden", "reference_kats.json")))
 
 
-@pytest.fixture(scope="module")
-def shim():
-    path = os.path.join(HERE, "cpp", "libreference_shim.so")
-    if not os.path.exists(path):
-        subprocess.check_call(["make", "-C", os.path.join(HERE, "cpp"), "libreference_shim.so"],
-                              stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+# the second build allows fused multiply-add wherever the compiler likes (-mfma
+# -ffp-contract=fast): the header has to keep its float loop free of it by itself
+@pytest.fixture(scope="module", params=["libreference_shim.so", "libreference_shim_fma.so"])
+def shim(request):
+    path = os.path.join(HERE, "cpp", request.param)
+    subprocess.check_call(["make", "-C", os.path.join(HERE, "cpp"), request.param],
+                          stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
     lib = ctypes.CDLL(path)
     vp, sz, f = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float
     lib.reference_gemm.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, sz, sz, sz, ctypes.c_int,

@@ -3,14 +3,17 @@
 (ccglib_pipeline_create + ccglib_pipeline_run) on the same buffers, two calls in a row, the
 second with a smaller input, so that what the first call left in the array is still there.
 Integer results bit for bit; float results bit for bit where the object takes the same route
-(transposes, then the tiled kernel) and within the float bounds of the oracle elsewhere."""
+(transposes, then the tiled kernel) and within the float bounds of the oracle elsewhere.
+The device's free memory is read on either side of every stateless call and must not move,
+and the call is captured into a HIP graph and replayed."""
 import numpy as np
 import pytest
 import torch
 
 import ccglib_amd as cc
 import oracle as orc
-from gpu_util import ORC_TYPE, check_float, dequantize, quantize, stream, to_device, to_host
+from gpu_util import (ORC_TYPE, capture_and_replay, check_float, dequantize, quantize, stream,
+                      to_device, to_host)
 
 pytestmark = pytest.mark.gpu
 
@@ -48,9 +51,13 @@ def _both(B, M, N, K, tin, tout, axis, c_axis, c_order, variant, alpha, beta, se
     pipe = cc.Pipeline(B, M, N, K, 0, stream(), axis, c_axis, ROW, COL, c_order, tin, tout, variant,
                        alpha, beta)
     pipe.Run(d_a.data_ptr(), d_b.data_ptr(), d_c1.data_ptr())
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]      # hipMemGetInfo: the device's, not torch's pool
     cc.pipeline_run_static(B, M, N, K, 0, stream(), axis, c_axis, ROW, COL, c_order, tin, tout,
                            variant, alpha, beta, d_a.data_ptr(), d_b.data_ptr(), d_c2.data_ptr())
+    free_enqueued = torch.cuda.mem_get_info()[0]
     torch.cuda.synchronize()
+    assert free_enqueued == free_before and torch.cuda.mem_get_info()[0] == free_before
     return to_host(d_c1, OUT_NP[tout]), to_host(d_c2, OUT_NP[tout])
 
 
@@ -109,7 +116,42 @@ def test_static_pipeline_against_oracle():
     check_float(to_host(d_c, np.float32).reshape(want.shape), want, w64, VT.float16, VT.float32)
 
 
+class _StaticCall:
+    """pipeline_run_static behind the Run(a, b, c) of an object, for capture_and_replay."""
+
+    def __init__(self, stream_handle, *dims_and_layout):
+        self.stream, self.args = stream_handle, dims_and_layout
+
+    def Run(self, d_a, d_b, d_c):
+        B, M, N, K, axis, c_axis, tin, tout = self.args
+        cc.pipeline_run_static(B, M, N, K, 0, self.stream, axis, c_axis, ROW, COL, ROW, tin, tout,
+                               cc.Variant.opt, 1, 0, d_a, d_b, d_c)
+
+
+@pytest.mark.parametrize("tin,tout,axis", [(VT.float16, VT.float32, INTERLEAVED),
+                                           (VT.int1, VT.int32, PLANAR)])
+def test_static_pipeline_in_a_graph(tin, tout, axis):
+    """The callers this entry point is for: captured once, replayed on changed input, every
+    replay equal to the eager call."""
+    B, M, N, K = 3, 200, 330, 96
+    int1 = tin == VT.int1
+    a = torch.zeros(B * 2 * M * K, dtype=torch.uint8 if int1 else torch.float16, device="cuda")
+    b = torch.zeros(B * 2 * N * K, dtype=torch.uint8 if int1 else torch.float16, device="cuda")
+
+    def fill(r):
+        g = torch.Generator(device="cuda").manual_seed(300 + r)
+        for t in (a, b):
+            if int1:
+                t.copy_(torch.randint(0, 2, t.shape, generator=g, device="cuda", dtype=torch.uint8))
+            else:
+                t.copy_(torch.randn(t.shape, generator=g, device="cuda").to(torch.float16))
+
+    capture_and_replay(lambda s: _StaticCall(s, B, M, N, K, axis, PLANAR, tin, tout), [a, b], fill,
+                       (B * 2 * M * N,), torch.int32 if int1 else torch.float32)
+
+
 def test_static_pipeline_rejects_what_does_not_fit():
+    assert cc.static_scratch_bytes() == 32 << 20    # the default build
     # 2 x (2 x 4096 x 4096 x 2 bytes) of tiles = 128 MiB > the 32 MiB array: refused, nothing runs
     d = to_device(np.zeros(16, np.uint8))
     with pytest.raises(RuntimeError, match="static scratch"):
