@@ -271,7 +271,11 @@ CCGLIB_API int ccglib_pipeline_destroy(ccglib_pipeline_t pipeline);
  * work of create + run + destroy with that scratch in a static device array
  * of CCGLIB_AMD_STATIC_SCRATCH_BYTES, which every GPU the library's code is
  * loaded on holds until the process ends. It calls no hipMalloc / hipFree (nor
- * their stream-ordered forms) and creates no host objects.
+ * their stream-ordered forms) and creates no host objects. (The HIP runtime
+ * loads a code object on a GPU when something in it is first used there: the
+ * array comes to exist, and its bytes leave the device's free memory, at the
+ * first call on that GPU, which therefore belongs before a graph capture. No
+ * later call moves the device's free memory.)
  *   - Arguments as ccglib_pipeline_create followed by those of
  *     ccglib_pipeline_run; only enqueues on `stream`.
  *   - Route: [1-bit interleaved input: pack each batch] -> transpose A and B
