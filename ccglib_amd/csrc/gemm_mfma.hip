@@ -1984,15 +1984,15 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// The 192 x 256 block of gemm_mfma_wide.h (16-bit input, tiled layout): one
-// persistent block per compute unit.
-template <int DT, int TOUT>
+// The 192 x 256 block of gemm_mfma_wide.h (16-bit input; tiled layout, or IL: the
+// pipeline's interleaved rows): one persistent block per compute unit.
+template <int DT, int TOUT, bool IL = false>
 hipError_t launch_wide(const GemmParams &p, hipStream_t stream) {
   const KernelArgs a = make_kernel_args(p, kWideBX, kWideBY);
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_wide<DT, TOUT>;
+  auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL>;
   static std::atomic<bool> lds_allowed[kMaxDevices];
   if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
   const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
@@ -2024,9 +2024,18 @@ inline bool small_tiles_pay(const GemmParams &p, double penalty) {
 // outside C), but its tiles are 1.5 times as large, so more of the last round of
 // tiles can stay empty (8192^3: 5.4 rounds of 192 x 256 tiles against 8 full ones).
 inline bool wide_tiles_apply(const GemmParams &p) {
-  return p.variant == kOpt && !p.input_interleaved && !p.c_interleaved && !p.have_alpha &&
-         !p.have_beta && ((uintptr_t)p.c % 16 == 0) && p.nx % 64 == 0 && p.ny % 64 == 0 &&
-         p.k_tiles >= 2 && !p.k_in_memory;
+  if (p.c_interleaved || p.have_alpha || p.have_beta || (uintptr_t)p.c % 16 != 0 ||
+      p.nx % 64 != 0 || p.ny % 64 != 0 || p.k_in_memory) {
+    return false;
+  }
+  if (p.input_interleaved) {
+    // rows of whole 128-byte pieces (32 complex values), at least two of them; a
+    // lane's offset inside a copy of 8 rows is a 32-bit number
+    const size_t row_bytes = (size_t)2 * p.k * bits_of(p.type_in) / 8;
+    return bits_of(p.type_in) == 16 && row_bytes % 128 == 0 && row_bytes >= 256 &&
+           row_bytes < ((size_t)1 << 28) && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 16 == 0;
+  }
+  return p.variant == kOpt && p.k_tiles >= 2;
 }
 inline bool wide_tiles_pay(const GemmParams &p) {
   if (p.block_tile != 0) return p.block_tile == 3;
@@ -2056,6 +2065,9 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
     if constexpr (DT == kFloat32) {
       return hipErrorInvalidValue;
     } else if constexpr (KPM == 1) {
+      if constexpr (DtypeTraits<DT>::kElemBytes == 2) {
+        if (wide_tiles_apply(p) && wide_tiles_pay(p)) return launch_wide<DT, TOUT, true>(p, stream);
+      }
       if (small_tiles_pay(p, 1.15)) {
         return launch_dtl<DT, TOUT, 128, 128, 64, 32, 4, 2, kLoadInterleavedVec>(p, stream);
       }
@@ -2193,6 +2205,9 @@ const char *describe_gemm_mfma(const GemmParams &p) {
                              ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.y % 16 == 0);
   const double penalty = int1 ? 1.0 : bits8 ? 1.05 : 1.15;
   if (p.input_interleaved) {
+    if (bits16 && wide_tiles_apply(p) && wide_tiles_pay(p)) {
+      return "complex_gemm_mfma_wide, 192x256 block, one wave per SIMD, interleaved rows";
+    }
     return small_tiles_pay(p, penalty) ? "complex_gemm_mfma_dtl, 128x128 block, interleaved rows"
                                        : "complex_gemm_mfma_dtl, 256x128 block, interleaved rows";
   }

@@ -127,7 +127,21 @@ __device__ __forceinline__ TileCoord tile_coord_by_lane(const KernelArgs &args, 
 }
 
 
-template <int DT, int TOUT>
+// IL: the operands are the caller's rows of (re, im) pairs (the pipeline's
+// interleaved input), read in place. A K iteration then covers 128 bytes of every
+// row - 32 complex values, as with the two 64-byte planes of a tile - and, with k
+// running over the 64 numbers of such a piece,
+//   Re = sum (xr, -xi, ...) . (yr, yi, ...)     Im = sum (xi, xr, ...) . (yr, yi, ...)
+// so the Y fragments are used as they are and both variants of an X fragment
+// come from the raw one in registers (a sign flip of the odd elements, a swap
+// inside each pair: 16 vector instructions per 16 matrix instructions, two behind
+// each of a tile's last eight). The matrix instructions, the rings, the barrier
+// and the stores are those of the tiled layout. In LDS a slot is a sequence of 1 KiB
+// blocks of 8 rows, [the first 64 bytes of each row | the second 64 bytes]: a copy
+// instruction fetches 8 whole 128-byte lines, and every fragment read touches
+// the banks exactly as in the tiled layout (64-byte rows, 256 bytes apart every
+// four), so the chunk swizzles of that layout carry over.
+template <int DT, int TOUT, bool IL>
 __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArgs args) {
   static_assert(DtypeTraits<DT>::kTilesPerMfma == 1 && DtypeTraits<DT>::kElemBytes == 2,
                 "16-bit input");
@@ -139,13 +153,20 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   constexpr int Y_RING = XSLOTS * X_BYTES;
   // 1 KiB copies a wave issues per K tile: 6 row blocks of X and its own 8 of Y
   constexpr int kCopies = 14;
-  constexpr unsigned GROUP = 64 * kTileRowBytes;   // 64 rows of a slot
+  // 16 and 64 rows of a slot, and the distance from the first to the second
+  // fragment of a tile (im plane; second half of the 128 bytes)
+  constexpr unsigned TILE16 = IL ? 2048 : 16 * kTileRowBytes;
+  constexpr unsigned GROUP = 4 * TILE16;
+  constexpr unsigned X2ND = IL ? 512 : XP, Y2ND = IL ? 512 : YP;
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const unsigned k_tiles = args.k_tiles;
+  // (interleaved rows: the host counts 64-byte pieces and only launches this
+  // kernel for rows of whole 128-byte pieces)
+  const unsigned k_tiles = IL ? args.k_tiles / 2 : args.k_tiles;
+  const unsigned row_stride = 2 * args.row_stride_bytes;   // IL: bytes from row to row
   const unsigned total = args.blocks_x * args.blocks_y * args.batch;
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
 
@@ -188,13 +209,31 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   const int xt_row = 4 * (lane >> 4) + (((lane >> 2) & 3) ^ (lane >> 4));
   const unsigned lane_off_x_even = xt_row * kTileRowBytes + (lane & 3) * 16;
   const unsigned lane_off_x_odd = xt_row * kTileRowBytes + ((lane & 3) ^ 3) * 16;
+  // IL: lane L of a copy writes chunk position L & 3 of row slot (L >> 2) & 7 in
+  // half L >> 5 of an 8-row block. Y: row = slot, chunk XOR (row >> 1) & 3. X: the
+  // exchanged-roles order, in which slot 4 a + (i ^ a) of a 16-row block holds row
+  // 4 a + i and the chunks are XORed with 3 (16-row block & 1): for the 8-row block
+  // q = 6 wave + i of the slot that is a = 2 (i & 1) + (slot >> 2) and 16-row
+  // block parity ((i >> 1) + wave) & 1.
+  const int cs = (lane >> 2) & 7, ch = lane >> 5, cpos = lane & 3;
+  const unsigned il_off_y = cs * row_stride + (4 * ch + (cpos ^ ((cs >> 1) & 3))) * 16;
+  unsigned il_off_x[2][2];   // [i & 1][(i >> 1) & 1]
+#pragma unroll
+  for (int qp = 0; qp < 2; ++qp) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int a = 2 * qp + (cs >> 2), row = 4 * (cs >> 2) + ((cs & 3) ^ a);
+      const int bp = (e + wave) & 1;
+      il_off_x[qp][e] = row * row_stride + (4 * ch + (cpos ^ (3 * bp))) * 16;
+    }
+  }
 
   // Wave w copies the row blocks 6 (w & 1) .. + 5 of plane w / 2 of X (consecutive
   // KiB of the slot) and the 64 rows of Y that it multiplies (4 consecutive KiB in
   // either plane).
   const unsigned x_plane = wave >> 1, x_rb0 = 6 * (wave & 1);
   const unsigned x_lds = lds_base + x_plane * XP + x_rb0 * 1024;
-  const unsigned y_lds = lds_base + Y_RING + wave * 64 * kTileRowBytes;
+  const unsigned y_lds = lds_base + Y_RING + wave * (IL ? 64 * 128 : 64 * kTileRowBytes);
   struct Stream {
     unsigned n, kt;   // tile of the block and K tile of the request issued last
   };
@@ -204,6 +243,16 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   const char *x_src[6], *y_src = nullptr;
   auto point_x = [&](unsigned n) {
     const TileCoord tc = coords(n);
+    if constexpr (IL) {
+      const char *op = args.x + (size_t)tc.b * args.x_batch_bytes;
+#pragma unroll
+      for (int i = 0; i < 6; ++i) {
+        unsigned row0 = tc.block_x * BX + (6 * wave + i) * 8;
+        row0 = row0 < args.nx ? row0 : args.nx - 8;   // rows past the end: never stored
+        x_src[i] = op + (size_t)row0 * row_stride;
+      }
+      return;
+    }
     const char *op = args.x + (size_t)tc.b * args.x_batch_bytes + x_plane * kTilePlaneBytes;
 #pragma unroll
     for (int i = 0; i < 6; ++i) {
@@ -217,6 +266,11 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   auto point_y = [&](unsigned n) {
     const TileCoord tc = coords(n);
     const unsigned row0 = tc.block_y * BY + wave * 64;
+    if constexpr (IL) {
+      y_src = args.y + (size_t)tc.b * args.y_batch_bytes +
+              (size_t)(row0 < args.ny ? row0 : args.ny - 64) * row_stride;
+      return;
+    }
     unsigned tile = row0 / kTileRows;
     tile = tile < args.y_tiles ? tile : args.y_tiles - 1;
     y_src = args.y + (size_t)tc.b * args.y_batch_bytes +
@@ -227,6 +281,18 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // instruction occupies the compute unit's address unit for 16 cycles, and a wave
   // that issues the next one earlier waits - with its matrix instructions behind it.
   auto issue = [&](int c, unsigned x_slot, unsigned y_slot) {
+    if constexpr (IL) {
+      // 0 - 7: rows 8 c .. 8 c + 7 of the wave's 64 of Y; 8 - 13: its 8-row blocks of X
+      if (c < 8) {
+        load_1k_to_lds(y_src + (size_t)ys.kt * 128 + (size_t)(8 * c) * row_stride, il_off_y,
+                       y_lds + y_slot * Y_BYTES + c * 1024);
+      } else {
+        const int i = c - 8;
+        load_1k_to_lds(x_src[i] + (size_t)xs.kt * 128, il_off_x[i & 1][(i >> 1) & 1],
+                       x_lds + x_slot * X_BYTES + i * 1024);
+      }
+      return;
+    }
     if (c < 8) {
       const int plane = c >> 2, blk = c & 3;
       load_1k_to_lds(y_src + (size_t)ys.kt * kTileBytes + plane * kTilePlaneBytes + blk * 1024,
@@ -255,12 +321,16 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   auto rd = [](unsigned address) { return *reinterpret_cast<lds_int4_t *>(address); };
   const int r16 = lane & 15, g4 = lane >> 4;
   unsigned xo[4];   // X fragment of tile i of a 64-row group, inside a slot
+  // (IL: row slot S of a group lies at (S >> 3) KiB + 64 (S & 7) of the group's 8 KiB)
+  auto row_address = [](int slot) {
+    return IL ? (slot >> 3) * 1024 + (slot & 7) * 64 : slot * kTileRowBytes;
+  };
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    xo[i] = lds_base + (4 * r16 + (i ^ (r16 & 3))) * kTileRowBytes +
-            ((g4 ^ (3 * ((r16 >> 2) & 1))) * 16);
+    xo[i] = lds_base + row_address(4 * r16 + (i ^ (r16 & 3))) + ((g4 ^ (3 * ((r16 >> 2) & 1))) * 16);
   }
-  const unsigned yo = y_lds + swizzled_row_offset(r16, g4);
+  const unsigned yo = y_lds + (IL ? row_address(r16) + ((g4 ^ ((r16 >> 1) & 3)) * 16)
+                                  : swizzled_row_offset(r16, g4));
 
   // ---- pipeline ------------------------------------------------------------------
   point_x(0);
@@ -274,25 +344,59 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   for (int c = 0; c < kCopies; ++c) issue(c, 1, 1);
 
   unsigned x_slot = 0, y_slot = 0;   // slots of the current iteration
-  int4_t yr[4], yi[4];               // the Y fragments of the current K tile
-  int4_t xr[2], xi[2], xn[2];        // X fragments (re, im, -im) of the current and the next tile
-  auto flip = [](const int4_t &v) {
+  // the Y fragments of the current K tile (re and im; IL: first and second half of the 128 bytes)
+  int4_t yr[4], yi[4];
+  // X fragments of the current and the next tile: re, im, -im;
+  // IL: xr, xi the two halves with the odd elements negated, xn, xm the halves with
+  // the elements of each pair exchanged
+  int4_t xr[2], xi[2], xn[2], xm[2];
+  constexpr int kOddSign = (int)0x80000000u;
+  // Values derived from a fragment are taken by an empty asm statement where they
+  // are computed. Without it the compiler may sink the computation to just before
+  // the matrix instruction that reads the result (it does so across the branches
+  // around the C stores) - and for a matrix instruction in an asm statement it
+  // does not insert the wait states that such a read needs after a vector-ALU
+  // write: the instruction then sees the old register contents. With it, every
+  // derived value is written several matrix instructions before its first use.
+  auto swap_pairs = [](int v) {
+    int o = (int)__builtin_amdgcn_alignbit((unsigned)v, (unsigned)v, 16);
+    asm volatile("" : "+v"(o));
+    return o;
+  };
+  auto flip_sign = [](int v, int mask) {
+    int o = v ^ mask;
+    asm volatile("" : "+v"(o));
+    return o;
+  };
+  auto flip = [&](const int4_t &v) {
     int4_t o;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) o[w] = v[w] ^ (int)DtypeTraits<DT>::kSignMask;
+    for (int w = 0; w < 4; ++w) o[w] = flip_sign(v[w], (int)DtypeTraits<DT>::kSignMask);
     return o;
   };
   // what the last tile of "iteration -1" would have done for iteration 0
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies) : "memory");
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    yr[j] = rd(yo + j * 16 * kTileRowBytes);
-    yi[j] = rd(yo + YP + j * 16 * kTileRowBytes);
+    yr[j] = rd(yo + j * TILE16);
+    yi[j] = rd(yo + Y2ND + j * TILE16);
   }
   if constexpr (!kAblateBarrier) asm volatile("s_barrier" ::: "memory");
   xr[0] = rd(xo[0]);
-  xi[0] = rd(xo[0] + XP);
-  xn[0] = flip(xi[0]);
+  xi[0] = rd(xo[0] + X2ND);
+  if constexpr (IL) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      xn[0][w] = swap_pairs(xr[0][w]);
+      xm[0][w] = swap_pairs(xi[0][w]);
+      xr[0][w] = flip_sign(xr[0][w], kOddSign);
+      xi[0][w] = flip_sign(xi[0][w], kOddSign);
+    }
+    // (the first matrix instruction reads xr[0] right away)
+    asm volatile("s_nop 7" ::: "memory");
+  } else {
+    xn[0] = flip(xi[0]);
+  }
 
   float4_t acc_re[4][TX], acc_im[4][TX];
 
@@ -384,17 +488,38 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         if (p == 0) {
           const unsigned a = xo[(t + 1) & 3] + xa + ((t + 1) >> 2) * GROUP;
           xr[s ^ 1] = rd(a);
-          xi[s ^ 1] = rd(a + XP);
+          xi[s ^ 1] = rd(a + X2ND);
           CCGLIB_PIN;
         }
-        if (p >= 10 && p < 14) {
+        if (!IL && p >= 10 && p < 14) {
           // -im of the next tile, one instruction behind each of four MFMAs (four in a
           // row would hold up the next MFMA); pinned on both sides: moved up, it
           // would wait for the read just issued
           CCGLIB_PIN;
-          xn[s ^ 1][p - 10] = xi[s ^ 1][p - 10] ^ (int)DtypeTraits<DT>::kSignMask;
+          xn[s ^ 1][p - 10] = flip_sign(xi[s ^ 1][p - 10], (int)DtypeTraits<DT>::kSignMask);
           CCGLIB_PIN;
         }
+      }
+      if (IL && p >= 8) {
+        // both variants of the next tile's fragments (the next iteration's first
+        // tile behind the last one), two instructions behind each of eight MFMAs;
+        // the exchange reads the raw value, so it comes before the sign flip
+        const int ns = t + 1 < TX ? (s ^ 1) : 0, w = 2 * (p & 1);
+        CCGLIB_PIN;
+        if (p < 10) {
+          xn[ns][w] = swap_pairs(xr[ns][w]);
+          xn[ns][w + 1] = swap_pairs(xr[ns][w + 1]);
+        } else if (p < 12) {
+          xr[ns][w] = flip_sign(xr[ns][w], kOddSign);
+          xr[ns][w + 1] = flip_sign(xr[ns][w + 1], kOddSign);
+        } else if (p < 14) {
+          xm[ns][w] = swap_pairs(xi[ns][w]);
+          xm[ns][w + 1] = swap_pairs(xi[ns][w + 1]);
+        } else {
+          xi[ns][w] = flip_sign(xi[ns][w], kOddSign);
+          xi[ns][w + 1] = flip_sign(xi[ns][w + 1], kOddSign);
+        }
+        CCGLIB_PIN;
       }
       {
         // C stores behind every other MFMA (the odd ones; the copies go behind even
@@ -423,8 +548,16 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
       }
       if (t == TX - 1) {
         // The iteration boundary. MFMA 4 of the last tile has waited for the
-        // wave's last fragment read from this X slot.
-        if (p == 4) {
+        // wave's last fragment read from this X slot (IL: MFMA 0 has, whose operand
+        // was computed from it; the boundary is at MFMA 1 there, so that the two
+        // variants of the next fragments can be made behind MFMAs 8 - 15 as in
+        // every other tile - one copy of this iteration is then still to come).
+        constexpr int kBoundary = IL ? 1 : 4;
+        constexpr int kCopiesBefore = IL ? kCopies - 1 : kCopies;
+        static_assert(22 + 12 * (kCopiesBefore - 1) <= 16 * (TX - 1) + kBoundary &&
+                          (kCopiesBefore == kCopies || 22 + 12 * kCopiesBefore > 16 * (TX - 1) + kBoundary),
+                      "copies issued before the boundary");
+        if (p == kBoundary) {
           // This wave's copies of the next K tile are complete when nothing older
           // than the requests of this iteration is outstanding - which are its
           // copies and, in a first or last iteration of a tile that lies entirely
@@ -432,30 +565,31 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
           // not tell them from stores; where stores may have been skipped, the
           // smaller number is the safe one and waits for more than it has to).
           if ((CARRY || LAST) && target.all) {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies + kStoresPerIteration) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesBefore + kStoresPerIteration) : "memory");
           } else {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopies) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesBefore) : "memory");
           }
           // every wave's part of the next X tile has landed, and nobody reads the
           // current X slot any more
           if constexpr (!kAblateBarrier) asm volatile("s_barrier" ::: "memory");
           xr[0] = rd(xo[0] + xa_next);
-          xi[0] = rd(xo[0] + xa_next + XP);
-          yr[0] = rd(ya_next);
+          xi[0] = rd(xo[0] + xa_next + X2ND);
           CCGLIB_PIN;
         }
         // each Y fragment of the next K tile into the registers of its
-        // predecessor, behind that one's last use
-        if (p == 5) yr[1] = rd(ya_next + 16 * kTileRowBytes);
-        if (p == 6) yi[0] = rd(ya_next + YP);
-        if (p == 7) yi[1] = rd(ya_next + YP + 16 * kTileRowBytes);
-        if (p == 12) yr[2] = rd(ya_next + 32 * kTileRowBytes);
-        if (p == 13) yr[3] = rd(ya_next + 48 * kTileRowBytes);
-        if (p == 14) yi[2] = rd(ya_next + YP + 32 * kTileRowBytes);
-        if (p == 15) yi[3] = rd(ya_next + YP + 48 * kTileRowBytes);
-        if (p >= 5) CCGLIB_PIN;
-        if (p >= 12) {
-          xn[0][p - 12] = xi[0][p - 12] ^ (int)DtypeTraits<DT>::kSignMask;
+        // predecessor, behind that one's last use (in either order of the tile's
+        // matrix instructions)
+        if (p == 4) yr[0] = rd(ya_next);
+        if (p == 5) yr[1] = rd(ya_next + TILE16);
+        if (p == 6) yi[0] = rd(ya_next + Y2ND);
+        if (p == 7) yi[1] = rd(ya_next + Y2ND + TILE16);
+        if (p == 12) yr[2] = rd(ya_next + 2 * TILE16);
+        if (p == 13) yr[3] = rd(ya_next + 3 * TILE16);
+        if (p == 14) yi[2] = rd(ya_next + Y2ND + 2 * TILE16);
+        if (p == 15) yi[3] = rd(ya_next + Y2ND + 3 * TILE16);
+        if (p >= 4) CCGLIB_PIN;
+        if (!IL && p >= 12) {
+          xn[0][p - 12] = flip_sign(xi[0][p - 12], (int)DtypeTraits<DT>::kSignMask);
           CCGLIB_PIN;
         }
       }
@@ -471,6 +605,26 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     mfma16_asm<DT, false, Z>(ACC, Y, X);                                               \
   }                                                                                    \
   behind(t, P);
+      if constexpr (IL) {
+        // first half of the 128 bytes, then the second, for two Y tile rows at a time
+        CCGLIB_MM(acc_re[0][t], yr[0], xr[s], FIRST, 0)
+        CCGLIB_MM(acc_re[1][t], yr[1], xr[s], FIRST, 1)
+        CCGLIB_MM(acc_im[0][t], yr[0], xn[s], FIRST, 2)
+        CCGLIB_MM(acc_im[1][t], yr[1], xn[s], FIRST, 3)
+        CCGLIB_MM(acc_re[0][t], yi[0], xi[s], false, 4)
+        CCGLIB_MM(acc_re[1][t], yi[1], xi[s], false, 5)
+        CCGLIB_MM(acc_im[0][t], yi[0], xm[s], false, 6)
+        CCGLIB_MM(acc_im[1][t], yi[1], xm[s], false, 7)
+        CCGLIB_MM(acc_re[2][t], yr[2], xr[s], FIRST, 8)
+        CCGLIB_MM(acc_re[3][t], yr[3], xr[s], FIRST, 9)
+        CCGLIB_MM(acc_im[2][t], yr[2], xn[s], FIRST, 10)
+        CCGLIB_MM(acc_im[3][t], yr[3], xn[s], FIRST, 11)
+        CCGLIB_MM(acc_re[2][t], yi[2], xi[s], false, 12)
+        CCGLIB_MM(acc_re[3][t], yi[3], xi[s], false, 13)
+        CCGLIB_MM(acc_im[2][t], yi[2], xm[s], false, 14)
+        CCGLIB_MM(acc_im[3][t], yi[3], xm[s], false, 15)
+        continue;
+      }
       CCGLIB_MM(acc_re[0][t], yr[0], xr[s], FIRST, 0)
       CCGLIB_MM(acc_re[1][t], yr[1], xr[s], FIRST, 1)
       CCGLIB_MM(acc_im[0][t], yi[0], xr[s], FIRST, 2)

@@ -95,6 +95,8 @@ static const std::vector<Config> kConfigs = {
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
     {"f16 planar 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>, kFloat16, kFloat32, kLoadPlanarVec},
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
+    {"f16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32, true>, kFloat16, kFloat32, kLoadInterleavedVec},
+    {"bf16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32, true>, kBfloat16, kFloat32, kLoadInterleavedVec},
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
     {"fp8 interleaved 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
 };
@@ -459,7 +461,9 @@ int main(int argc, char **argv) {
     p.beta_im = 0;
     p.have_alpha = 0;
     p.have_beta = 0;
-    if (c.launch == launch_wide<kFloat16, kFloat32> || c.launch == launch_wide<kBfloat16, kFloat32>) {
+    if (c.launch == launch_wide<kFloat16, kFloat32> || c.launch == launch_wide<kBfloat16, kFloat32> ||
+        c.launch == launch_wide<kFloat16, kFloat32, true> ||
+        c.launch == launch_wide<kBfloat16, kFloat32, true>) {
       if (!wide_tiles_apply(p)) {
         std::printf("%-44s (not applicable to this shape)\n", c.name);
         continue;

@@ -408,3 +408,36 @@ def test_pipeline_planar_rows_read_in_place(tin, K, skew):
         host_c = np.full(B * 2 * M * N, np.nan, dtype=np.float32)
         p.RunHost(qa.ctypes.data, qb.ctypes.data, host_c.ctypes.data)
         assert np.array_equal(host_c, got.reshape(-1))
+
+
+@pytest.mark.parametrize("tin,tout", [(VT.float16, VT.float32), (VT.float16, VT.float16),
+                                      (VT.bfloat16, VT.float32), (VT.bfloat16, VT.bfloat16)])
+@pytest.mark.parametrize("c_order", [ROW, COL])
+def test_pipeline_interleaved_rows_wide_block(tin, tout, c_order):
+    """GEMM_BLOCK_TILE = 3 for 16-bit interleaved rows read in place: the 192 x 256 block
+    (planar C without alpha or beta, M and N multiples of 64, rows of whole 128-byte
+    pieces, i.e. K a multiple of 32) against the oracle, and bit for bit against the
+    256 x 128 block: tiles inside C and tiles of which only some 64-column groups or
+    64-row pieces are, two to many K pieces, more C tiles than compute units."""
+    for seed, (B, M, N, K) in enumerate([(2, 256, 192, 64), (3, 320, 448, 96), (2, 512, 832, 992),
+                                         (40, 256, 576, 64), (1, 64, 64, 128)]):
+        rng = np.random.default_rng(40 + seed)
+        qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), tin)
+        qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), tin)
+        d_a = to_device(np.ascontiguousarray(qa.transpose(0, 2, 3, 1)).reshape(-1))
+        d_b = to_device(np.ascontiguousarray(qb.transpose(0, 2, 3, 1)).reshape(-1))
+        out_np = np.float32 if tout == VT.float32 else np.uint16
+        results = []
+        for block_tile in (3, 1):
+            with cc.option(cc.Option.gemm_block_tile, block_tile):
+                p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, c_order, tin, tout,
+                                cc.Variant.opt)
+            d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32) if tout == VT.float32
+                            else np.full(B * 2 * M * N, 0x7fc0, dtype=np.uint16))
+            p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
+            torch.cuda.synchronize()
+            results.append(to_host(d_c, out_np))
+        want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], int(c_order))
+        w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], int(c_order))
+        check_float(dequantize(results[0], tout).reshape(want.shape), dequantize(want, tout), w64, tin, tout)
+        assert np.array_equal(results[0], results[1]), (B, M, N, K)
