@@ -94,6 +94,7 @@ class Option(enum.IntEnum):
     host_chunk_bytes = 2
     gemm_block_tile = 3
     expect_unaligned = 4
+    pipeline_route = 5
 
 
 def set_option(option, value):
@@ -235,6 +236,13 @@ class Pipeline(_Handle):
 
     def Run(self, d_a, d_b, d_c):
         _capi.check(_capi.load().ccglib_pipeline_run(self._h, _ptr(d_a), _ptr(d_b), _ptr(d_c)))
+
+    def ReadsInPlace(self):
+        """Whether the GEMM of this pipeline reads the caller's rows in place (no transposes);
+        no counterpart in the reference (see Option.pipeline_route)."""
+        out = ctypes.c_int(0)
+        _capi.check(_capi.load().ccglib_pipeline_reads_in_place(self._h, ctypes.byref(out)))
+        return bool(out.value)
 
     def RunHost(self, h_a, h_b, h_c):
         _capi.check(_capi.load().ccglib_pipeline_run_host(self._h, _ptr(h_a), _ptr(h_b),

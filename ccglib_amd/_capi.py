@@ -36,6 +36,7 @@ SIGNATURES = {
                                     _i, _f, _f, _f, _f]),
     "ccglib_pipeline_run": (_i, [_vp, _vp, _vp, _vp]),
     "ccglib_pipeline_run_host": (_i, [_vp, _vp, _vp, _vp]),
+    "ccglib_pipeline_reads_in_place": (_i, [_vp, ctypes.POINTER(_i)]),
     "ccglib_pipeline_destroy": (_i, [_vp]),
     "ccglib_pipeline_run_static": (_i, [_sz, _sz, _sz, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                         _f, _f, _f, _f, _vp, _vp, _vp]),

@@ -178,7 +178,7 @@ struct ccglib_pipeline {
 namespace {
 
 // Process-wide options (ccglib_amd_set_option), read when an object is created.
-size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0, 0, 0};
+size_t g_options[CCGLIB_AMD_OPTION_COUNT] = {0, 1, 0, 0, 0, 0};
 
 // Largest buffer of 1-bit tiles a pipeline allocates; beyond it the pipeline
 // runs the reference's sequence of kernels on its packed / transposed buffers.
@@ -340,6 +340,9 @@ int ccglib_amd_set_option(int option, size_t value) {
   }
   if (option == CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE && value > 3) {
     return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "GEMM_BLOCK_TILE is 0, 1, 2 or 3 (got %zu)", value);
+  }
+  if (option == CCGLIB_AMD_OPTION_PIPELINE_ROUTE && value > 2) {
+    return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "PIPELINE_ROUTE is 0, 1 or 2 (got %zu)", value);
   }
   g_options[option] = value;
   return CCGLIB_OK;
@@ -801,23 +804,43 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
   // GEMM as it is (the kernel de-interleaves in its arithmetic), which saves the
   // two transposes and their intermediate buffers for either variant.
   const size_t in_bits = (size_t)bits_of(input_type);
-  // Reading rows in place costs the GEMM 6-9 % against reading tiles; the
-  // transposes cost two bandwidth-bound passes over A and B. The first is the
-  // smaller price while M N / (M + N) stays below about 2800 (16-bit) or 3000
-  // (8-bit input), from the measured rates of the kernels involved.
+  // Reading rows in place costs the GEMM a few per cent against reading tiles; the
+  // transposes cost two bandwidth-bound passes over A and B and two more launches.
+  // The GEMM's work grows with M N and the transposes' with M + N, so reading in
+  // place is the smaller price while
+  //   M N / (M + N)  <  T (1 + c / (B K (M + N)))
+  // with the break-even T of large problems and c the launches' fixed cost in
+  // operand elements. Measured (python -m ccglib_amd.tuning.pipeline_crossover at
+  // K = 256, 1024, 4096): 16-bit interleaved rows T = 3800 where the 192 x 256 kernel
+  // reads them (planar C, no alpha / beta, M and N multiples of 64, K of 32) and
+  // 2800 elsewhere, 8-bit interleaved rows T = 2700, c = 1e7 for both.
   const double mn_over_sum = (M + N) ? (double)M * (double)N / (double)(M + N) : 0.0;
+  const double operand_elements = (double)B * (double)K * (double)(M + N);
+  // (option PIPELINE_ROUTE: 1 in place wherever possible, 2 never for the opt variant)
+  const size_t route = g_options[CCGLIB_AMD_OPTION_PIPELINE_ROUTE];
+  auto below = [&](double break_even, double fixed_cost) {
+    return route == 1 ||
+           (route == 0 && operand_elements > 0 &&
+            mn_over_sum < break_even * (1.0 + fixed_cost / operand_elements));
+  };
+  const bool wide_rows = in_bits == 16 && output_complex_axis_location == kPlanar &&
+                         alpha_re == 1.f && alpha_im == 0.f && beta_re == 0.f && beta_im == 0.f &&
+                         M % 64 == 0 && N % 64 == 0 && K % 32 == 0 && K >= 64;
   const bool fused = allow_fused && !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&
-                     (variant == kBasic || mn_over_sum < (in_bits == 16 ? 2800.0 : 3000.0));
+                     (variant == kBasic ||
+                      below(in_bits == 8 ? 2700.0 : wide_rows ? 3800.0 : 2800.0, 1.0e7));
   // Planar input of the opt variant whose rows are whole 16-byte chunks: the GEMM
   // can read the rows in place as well (the basic variant's loader, same
-  // arithmetic and K order as on tiles). That costs the GEMM 9-12 %, so the
-  // break-even against the two transposes lies lower, at about 1750.
+  // arithmetic and K order as on tiles). That costs the GEMM more (the tiled
+  // operands have the 192 x 256 kernel), so the break-even lies lower: T = 1500,
+  // c = 6e6 (measured on squares; long rectangles at small K would still gain up to
+  // 8 % from reading in place beyond it).
   const bool planar_in_place = allow_fused && !packing && variant == kOpt &&
                                input_complex_axis_location == kPlanar &&
                                output_complex_axis_location == kPlanar && K > 0 &&
                                (in_bits == 8 || in_bits == 16 || in_bits == 32) &&
-                               (K * in_bits / 8) % 16 == 0 && mn_over_sum < 1750.0;
+                               (K * in_bits / 8) % 16 == 0 && below(1500.0, 6.0e6);
   // The reference transposes for the opt variant only (:53) and hands interleaved
   // input of the basic variant to a kernel that reads it as planar. Here such
   // input is always de-interleaved: in the GEMM's loader (fused) or, where that
@@ -947,6 +970,12 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
 }  // namespace
 
 extern "C" {
+
+int ccglib_pipeline_reads_in_place(ccglib_pipeline_t p, int *in_place) {
+  if (!p || !in_place) return fail(CCGLIB_ERROR_INVALID_ARGUMENT, "null argument");
+  *in_place = p->fused ? 1 : 0;
+  return CCGLIB_OK;
+}
 
 int ccglib_pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, size_t K,
                            int device, void *stream, int input_complex_axis_location,

@@ -455,10 +455,12 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     if constexpr (kAblateStores) {
       if (v[0] == 12345.678f) *reinterpret_cast<Tout *>(p) = (Tout)v[1];   // (timing-only build)
     } else if constexpr (TOUT == kFloat32) {
-      *reinterpret_cast<float4_t *>(p) = float4_t{v[0], v[1], v[2], v[3]};
+      // (C is written once and not read again by this kernel: stores marked
+      // non-temporal measured 0.4 % faster at B=64 512x4096x576)
+      __builtin_nontemporal_store(float4_t{v[0], v[1], v[2], v[3]}, reinterpret_cast<float4_t *>(p));
     } else {
       Tout t4[4] = {(Tout)v[0], (Tout)v[1], (Tout)v[2], (Tout)v[3]};
-      *reinterpret_cast<ushort4_t *>(p) = __builtin_bit_cast(ushort4_t, t4);
+      __builtin_nontemporal_store(__builtin_bit_cast(ushort4_t, t4), reinterpret_cast<ushort4_t *>(p));
     }
   };
   constexpr int kStoresPerIteration = 48;

@@ -28,8 +28,15 @@
 // two matrix instructions costs a wave that has the SIMD to itself, the rate of a
 // plain fill of 1 GiB, and the rate at which all compute units read a window of a
 // given size over and over (L2 and memory-side cache).
+// TUNE_GEMM_SMALL (make SMALL=1): only the 16-bit rows of the beamformer sweep - the
+// kernels one works on most - for a build of under a minute.
+#ifdef TUNE_GEMM_SMALL
+#define CCGLIB_GEMM_MFMA_PART 99   // none of the library's own instantiations
+#endif
 #include "../csrc/gemm_mfma.hip"
+#ifndef TUNE_GEMM_SMALL
 #include "../csrc/gemm_int1.hip"
+#endif
 
 #include <hip/hip_fp8.h>
 
@@ -60,28 +67,33 @@ struct Config {
   double peak = 0;           // what "of peak" refers to (0: the input type's MFMA peak)
 };
 
+#ifndef TUNE_GEMM_SMALL
 // the 1-bit GEMM on the vector ALUs (XOR + population count), whatever the layout
 static hipError_t launch_popcount(const GemmParams &p, hipStream_t stream) {
   GemmParams q = p;
   q.int1_direct = 0;
   return launch_gemm_int1(q, stream);
 }
+#endif
 // 256 CUs x 64 lane-operations per clock x 2.4 GHz, 8 lane-operations (4 XOR, 4
 // counts) per 32 complex products of 8 "operations" each
 constexpr double kPopcountRoof = 256 * 64 * 2.4e9 * 32 / 1e12;   // 1258 TOP/s
 
 // name: type, [operand layout,] block BX x BY, wave WX x WY, ring slots, MFMA rows
 static const std::vector<Config> kConfigs = {
+#ifndef TUNE_GEMM_SMALL
     {"f16 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat16, kFloat32},
+#endif
     {"f16 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 y3 x4 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true, 4>, kFloat16, kFloat32},
     {"f16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32>, kFloat16, kFloat32},
+    {"bf16 256x128 w64x64 s3 m16 xt", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kBfloat16, kFloat32},
+    {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32>, kBfloat16, kFloat32},
+#ifndef TUNE_GEMM_SMALL
     {"f16 256x128 w64x64 s3 m32", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat16, kFloat32},
     {"f16 128x128 w64x64 s2 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 16>, kFloat16, kFloat32},
     {"f16 128x128 w64x32 s4 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 32, 4, 2, kLoadTiled, 16>, kFloat16, kFloat32},
-    {"bf16 256x128 w64x64 s3 m16 xt", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kBfloat16, kFloat32},
-    {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32>, kBfloat16, kFloat32},
     {"f32 256x128 w64x64 s3 m16", launch_dtl<kFloat32, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16>, kFloat32, kFloat32},
     {"fp8 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
     {"fp8 128x128 w64x64 s2 m32", launch_dtl<kFloat8e4m3, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 32>, kFloat8e4m3, kFloat32},
@@ -91,14 +103,23 @@ static const std::vector<Config> kConfigs = {
     // the 1-bit GEMM on the vector ALUs; "of peak" is of its issue roof
     {"int1 popcount 128x128 (vector ALU)", launch_popcount, kInt1, kInt32, kLoadTiled, kPopcountRoof},
     {"int1 popcount planar 128x128 (vector ALU)", launch_popcount, kInt1, kInt32, kLoadPlanarVec, kPopcountRoof},
+#endif
     // planar rows (basic variant) and raw interleaved rows (the pipeline's fused mode)
+#ifndef TUNE_GEMM_SMALL
     {"f16 planar 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16>, kFloat16, kFloat32, kLoadPlanarVec},
+#endif
+#ifndef TUNE_GEMM_SMALL
     {"f16 planar 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 16, true>, kFloat16, kFloat32, kLoadPlanarVec},
+#endif
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"f16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32, true>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"bf16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32, true>, kBfloat16, kFloat32, kLoadInterleavedVec},
+#ifndef TUNE_GEMM_SMALL
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
+#endif
+#ifndef TUNE_GEMM_SMALL
     {"fp8 interleaved 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 32>, kFloat8e4m3, kFloat32, kLoadInterleavedVec},
+#endif
 };
 
 static double peak_of(int type) {

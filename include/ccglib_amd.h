@@ -91,7 +91,9 @@ CCGLIB_API const char *ccglib_version(void);
  *                    without alpha or beta, M and N multiples of 64, K of more
  *                    than 32) when those fill the compute units well enough;
  *                    1: always 256 x 128; 2: always 128 x 128; 3: 192 x 256
- *                    wherever that kernel applies, else as 0.
+ *                    wherever that kernel applies, else as 0. The 192 x 256
+ *                    block also serves 16-bit interleaved rows read in place
+ *                    (the pipeline) when K is a multiple of 32.
  *   EXPECT_UNALIGNED 0 (default): a basic-variant GEMM that meets operands that
  *                    are not 16-byte aligned allocates its tiled copies at that
  *                    Run, and a pipeline that reads rows in place creates the
@@ -101,6 +103,14 @@ CCGLIB_API const char *ccglib_version(void);
  *                    registers, the pipeline reports an error); 1: both are
  *                    allocated when the object is created, and no device Run
  *                    allocates.
+ *   PIPELINE_ROUTE   0 (default): an opt-variant pipeline whose input rows are
+ *                    whole 16-byte chunks lets the GEMM read them in place
+ *                    where that is faster than transposing them into tiles
+ *                    first (small M N / (M + N); the break-even points are
+ *                    measured ones), and transposes otherwise; 1: in place
+ *                    wherever the GEMM can; 2: always through the transposes.
+ *                    ccglib_pipeline_reads_in_place tells which one an object
+ *                    took.
  * ---------------------------------------------------------------------- */
 enum {
   CCGLIB_AMD_OPTION_INT1_POPCOUNT = 0,
@@ -108,7 +118,8 @@ enum {
   CCGLIB_AMD_OPTION_HOST_CHUNK_BYTES = 2,
   CCGLIB_AMD_OPTION_GEMM_BLOCK_TILE = 3,
   CCGLIB_AMD_OPTION_EXPECT_UNALIGNED = 4,
-  CCGLIB_AMD_OPTION_COUNT = 5
+  CCGLIB_AMD_OPTION_PIPELINE_ROUTE = 5,
+  CCGLIB_AMD_OPTION_COUNT = 6
 };
 CCGLIB_API int ccglib_amd_set_option(int option, size_t value);
 CCGLIB_API int ccglib_amd_get_option(int option, size_t *value);
@@ -260,6 +271,11 @@ CCGLIB_API int ccglib_pipeline_run(ccglib_pipeline_t pipeline, const void *d_a,
 CCGLIB_API int ccglib_pipeline_run_host(ccglib_pipeline_t pipeline,
                                         const void *h_a, const void *h_b,
                                         void *h_c);
+/* Whether the object's GEMM reads the caller's rows in place (1) or the tiles
+ * that its transposes write (0); see the option PIPELINE_ROUTE. No counterpart
+ * in the reference, which always transposes for the opt variant
+ * (src/pipeline/Pipeline.cpp:53, :78-93). */
+CCGLIB_API int ccglib_pipeline_reads_in_place(ccglib_pipeline_t pipeline, int *in_place);
 CCGLIB_API int ccglib_pipeline_destroy(ccglib_pipeline_t pipeline);
 
 /* ------------------------------------------------------------------------

@@ -320,16 +320,18 @@ def test_pipeline_interleaved_input(tin, tout, K, variant):
 
 
 @pytest.mark.parametrize("tin", [VT.float16, VT.float8e4m3])
-def test_pipeline_interleaved_input_large_c(tin):
-    # With M N / (M + N) above about 2800 (3000 for 8-bit input) the opt pipeline transposes
-    # interleaved input into tiles instead of reading the rows in place (the GEMM then runs
-    # enough faster to pay for the two transposes); same numbers either way.
-    B, M, N, K = 1, 6144, 6144, 64      # M N / (M + N) = 3072
+@pytest.mark.parametrize("route", [1, 2])
+def test_pipeline_interleaved_input_either_route(tin, route):
+    # The opt pipeline reads interleaved rows in place or transposes them into tiles first,
+    # whichever it expects to be faster (option PIPELINE_ROUTE forces one): same numbers.
+    B, M, N, K = 1, 6144, 6144, 64
     rng = np.random.default_rng(31)
     qa = quantize(rng.uniform(-1, 1, B * 2 * M * K), tin)
     qb = quantize(rng.uniform(-1, 1, B * 2 * N * K), tin)
-    p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, tin, VT.float32,
-                    cc.Variant.opt)
+    with cc.option(cc.Option.pipeline_route, route):
+        p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, ROW, tin, VT.float32,
+                        cc.Variant.opt)
+    assert p.ReadsInPlace() == (route == 1)
     d_a, d_b = to_device(interleaved(qa, B, M, K)), to_device(interleaved(qb, B, N, K))
     d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32))
     p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
@@ -337,6 +339,61 @@ def test_pipeline_interleaved_input_large_c(tin):
     got = to_host(d_c, np.float32).reshape(B, 2, M, N)
     want = orc.gemm(qa, qb, M, N, K, ORC_TYPE[tin], orc.FLOAT32)
     check_float(got, want, orc.gemm_float64(qa, qb, M, N, K, ORC_TYPE[tin]), tin, VT.float32)
+
+
+def _time_runs(pipe, a, b, c, budget_ms=30.0):
+    cur = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        pipe.Run(a.data_ptr(), b.data_ptr(), c.data_ptr())
+    e0.record(cur)
+    pipe.Run(a.data_ptr(), b.data_ptr(), c.data_ptr())
+    e1.record(cur)
+    e1.synchronize()
+    n = max(3, int(budget_ms / max(e0.elapsed_time(e1), 1e-3)))
+    e0.record(cur)
+    for _ in range(n):
+        pipe.Run(a.data_ptr(), b.data_ptr(), c.data_ptr())
+    e1.record(cur)
+    e1.synchronize()
+    return e0.elapsed_time(e1) / n
+
+
+@pytest.mark.parametrize("tin,tdt,axis", [(VT.float16, torch.float16, INTERLEAVED),
+                                          (VT.float8e4m3, torch.float8_e4m3fn, INTERLEAVED),
+                                          (VT.float16, torch.float16, PLANAR)])
+def test_pipeline_takes_the_faster_route(tin, tdt, axis):
+    """Either side of the break-even points in ccglib_pipeline_create (the sweep behind them:
+    python -m ccglib_amd.tuning.pipeline_crossover): the route the default takes is timed
+    against the other one (PIPELINE_ROUTE = 1 / 2, best of three alternations of about 30 ms
+    each) and may be at most 5 % slower."""
+    K = 1024
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    taken = []
+    for M, N in [(512, 4096), (2048, 2048), (3072, 3072), (5120, 5120), (8192, 8192), (12288, 12288)]:
+        B = max(1, (1 << 27) // (M * N))
+        il = axis == INTERLEAVED
+        scale = 448.0 / 5.8 if tin == VT.float8e4m3 else 1.0
+        a = (torch.randn((B, M, K, 2) if il else (B, 2, M, K), device="cuda", generator=gen) * scale).to(tdt)
+        b = (torch.randn((B, N, K, 2) if il else (B, 2, N, K), device="cuda", generator=gen) * scale).to(tdt)
+        c = torch.empty((B, 2, M, N), device="cuda")
+        pipes = {}
+        for route in (0, 1, 2):
+            with cc.option(cc.Option.pipeline_route, route):
+                pipes[route] = cc.Pipeline(B, M, N, K, 0, stream(), axis, PLANAR, ROW, COL, ROW, tin,
+                                           VT.float32, cc.Variant.opt)
+        assert pipes[1].ReadsInPlace() and not pipes[2].ReadsInPlace()
+        best = {1: float("inf"), 2: float("inf")}
+        for _ in range(3):
+            for route in (1, 2):
+                best[route] = min(best[route], _time_runs(pipes[route], a, b, c))
+        chosen = 1 if pipes[0].ReadsInPlace() else 2
+        taken.append(chosen)
+        print("%s %s %dx%d: in place %.4f ms, transposed %.4f ms, default %s" % (
+            tin.name, axis.name, M, N, best[1], best[2], "in place" if chosen == 1 else "transposed"), flush=True)
+        assert best[chosen] <= 1.05 * best[3 - chosen], (M, N, best)
+        del pipes, a, b, c
+    assert taken[0] == 1 and taken[-1] == 2     # the sweep crosses the break-even point
 
 
 def test_pipeline_basic_rejects_interleaved_output():
