@@ -249,11 +249,40 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
         per_kernel[label + "_ms"] = ms
         per_kernel[label + "_gbs"] = nbytes / ms / 1e6
         per_kernel[label + "_frac_of_hbm_peak"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
+    # What an event pair adds to the interval it brackets: 20 empty intervals on the same
+    # stream. (The in-step figures contain it once per interval; the back-to-back ones
+    # spread it over 20 launches.)
+    empty = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+    for e in empty:
+        e.record()
+    empty[-1].synchronize()
+    overhead_ms = sum(empty[i].elapsed_time(empty[i + 1]) for i in range(20)) / 20
+    per_kernel["event_interval_overhead_ms"] = overhead_ms
+    for label, _, nbytes in kernels:
+        net = per_kernel[label + "_ms"] - overhead_ms
+        if net > 0:
+            per_kernel[label + "_frac_net_of_event_overhead"] = nbytes / net / 1e6 / HBM_PEAK_GBS
+    # Two launches of the same kernel on operands of different size give its fixed cost per
+    # launch and its asymptotic rate: ms = fixed + bytes / rate.
+    sizes = {label: nbytes for label, _, nbytes in standalone}
+    if "transpose_a" in sizes and "transpose_b" in sizes and \
+            max(sizes["transpose_a"], sizes["transpose_b"]) >= 2 * min(sizes["transpose_a"], sizes["transpose_b"]):
+        (la, lb) = ("transpose_a", "transpose_b") if sizes["transpose_a"] < sizes["transpose_b"] else \
+            ("transpose_b", "transpose_a")
+        rate = (sizes[lb] - sizes[la]) / (per_kernel[lb + "_ms"] - per_kernel[la + "_ms"])   # bytes per ms
+        fixed_ms = per_kernel[la + "_ms"] - sizes[la] / rate
+        per_kernel["transpose_launch_fixed_cost_us"] = fixed_ms * 1e3
+        per_kernel["transpose_asymptotic_gbs"] = rate / 1e6
+        per_kernel["transpose_asymptotic_frac_of_hbm_peak"] = rate / 1e6 / HBM_PEAK_GBS
     per_kernel["method"] = ("gemm, transposes (both operands through ccglib_transpose_run_pair: one "
                             "launch when one operand is small, else two) and packing_*: event pairs "
                             "inside the timed steps; transpose_a / transpose_b / "
                             "transposes_back_to_back (the pair call again): 20 back to back between "
-                            "two events after the steps")
+                            "two events after the steps; event_interval_overhead_ms: what an empty "
+                            "interval between two events measures on this stream (contained once in "
+                            "every in-step figure; *_frac_net_of_event_overhead subtracts it); "
+                            "transpose_launch_fixed_cost_us / transpose_asymptotic_*: from the two "
+                            "stand-alone transposes of different size, ms = fixed + bytes / rate")
 
     # (the library says which of its kernels the GEMM object launches)
     kernel_name = "%s <%s -> %s>" % (gemm.KernelName(), tin_name, tout_name)
