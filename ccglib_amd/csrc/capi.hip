@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -114,8 +115,11 @@ struct ccglib_gemm {
   // and B are first copied into the tiled layout (A at the start of
   // `workspace`, B at retile_b_offset) and the kernel of the opt variant runs on
   // the copies. retile_allowed: the option was on when the object was created.
-  bool retile = false, retile_allowed = true;
+  // (retile is set once, possibly by a Run: under lazy_lock, and read without it)
+  std::atomic<bool> retile{false};
+  bool retile_allowed = true;
   size_t retile_b_offset = 0;
+  std::mutex lazy_lock;
   // 1-bit GEMM: the MFMA kernel multiplies the packed words (0: the option that
   // keeps it on the vector ALUs was set when the object was created)
   int int1_direct = 1;
@@ -152,7 +156,8 @@ struct ccglib_pipeline {
   // `unfused` is the pipeline with transposes that takes over for buffers that
   // are not 16-byte aligned, created by the first Run that meets such buffers
   bool fused = false;
-  ccglib_pipeline *unfused = nullptr;
+  std::atomic<ccglib_pipeline *> unfused{nullptr};   // (set once, under lazy_lock)
+  std::mutex lazy_lock;
   ccglib_packing_t pack_a = nullptr, pack_b = nullptr;
   ccglib_transpose_t trans_a = nullptr, trans_b = nullptr;
   ccglib_gemm_t gemm = nullptr;
@@ -203,8 +208,8 @@ void make_retile_workspace(ccglib_gemm *g) {
   DeviceGuard guard(g->device);
   if (guard.status() == hipSuccess && hipMalloc(&g->workspace, bytes_a + bytes_b) == hipSuccess) {
     g->workspace_bytes = bytes_a + bytes_b;
-    g->retile = true;
     g->retile_b_offset = bytes_a;
+    g->retile.store(true, std::memory_order_release);
   } else {
     g->workspace = nullptr;
     (void)hipGetLastError();
@@ -442,8 +447,12 @@ int ccglib_gemm_run(ccglib_gemm_t g, const void *d_a, const void *d_b, void *d_c
     // captured into a graph, where the kernel that reads such rows through
     // registers runs instead (the option EXPECT_UNALIGNED makes the object
     // allocate at construction).
-    if (misaligned && !g->retile && !stream_is_capturing(g->stream)) make_retile_workspace(g);
-    retile_now = g->retile && (misaligned || row_bytes % 16 != 0);
+    if (misaligned && !g->retile.load(std::memory_order_acquire) && !stream_is_capturing(g->stream)) {
+      // (two threads may Run one object: only one of them allocates)
+      std::lock_guard<std::mutex> lock(g->lazy_lock);
+      make_retile_workspace(g);
+    }
+    retile_now = g->retile.load(std::memory_order_acquire) && (misaligned || row_bytes % 16 != 0);
   }
   if (retile_now) {
     TransposeParams t;
@@ -745,7 +754,7 @@ int ccglib_pipeline_destroy(ccglib_pipeline_t p) {
     if (p->d_b_trans) (void)hipFree(p->d_b_trans);
   }
   destroy_host_lanes(p);
-  ccglib_pipeline_destroy(p->unfused);
+  ccglib_pipeline_destroy(p->unfused.load());
   ccglib_packing_destroy(p->pack_a);
   ccglib_packing_destroy(p->pack_b);
   ccglib_transpose_destroy(p->trans_a);
@@ -951,10 +960,12 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
         g_options[CCGLIB_AMD_OPTION_EXPECT_UNALIGNED] != 0) {
       // the pipeline with transposes that takes over for unaligned buffers, now
       // rather than at the first Run that meets them
-      rc = pipeline_create(&p->unfused, B, M, N, K, device, stream, input_complex_axis_location,
+      ccglib_pipeline *stand_by = nullptr;
+      rc = pipeline_create(&stand_by, B, M, N, K, device, stream, input_complex_axis_location,
                            output_complex_axis_location, a_mem_order, b_mem_order, c_mem_order,
                            input_type, output_type, variant, alpha_re, alpha_im, beta_re, beta_im,
                            false);
+      p->unfused.store(stand_by, std::memory_order_release);
     }
   } while (false);
   if (rc != CCGLIB_OK) {
@@ -996,19 +1007,26 @@ int ccglib_pipeline_run(ccglib_pipeline_t p, const void *d_a, const void *d_b, v
     // The GEMM's copies to LDS need 16-byte aligned rows; the transposes take any
     // element-aligned address. The pipeline that runs them is created here, once
     // (the one allocation a device Run may make), and kept.
-    if (!p->unfused) {
+    ccglib_pipeline *stand_by = p->unfused.load(std::memory_order_acquire);
+    if (!stand_by) {
       if (stream_is_capturing(p->stream)) {
         return fail(CCGLIB_ERROR_INVALID_ARGUMENT,
                     "pipeline input is not 16-byte aligned: the pipeline with transposes that takes "
                     "such buffers cannot be allocated while the stream is being captured (run once "
                     "before the capture, or create the pipeline with the option EXPECT_UNALIGNED)");
       }
-      rc = pipeline_create(&p->unfused, p->B, p->M, p->N, p->K, p->device, p->stream, p->in_axis,
-                           p->c_axis, p->a_order, p->b_order, p->c_order, p->type_in, p->type_out,
-                           p->variant, p->alpha_re, p->alpha_im, p->beta_re, p->beta_im, false);
-      if (rc != CCGLIB_OK) return rc;
+      // (two threads may Run one object: only one of them creates the stand-by)
+      std::lock_guard<std::mutex> lock(p->lazy_lock);
+      stand_by = p->unfused.load(std::memory_order_acquire);
+      if (!stand_by) {
+        rc = pipeline_create(&stand_by, p->B, p->M, p->N, p->K, p->device, p->stream, p->in_axis,
+                             p->c_axis, p->a_order, p->b_order, p->c_order, p->type_in, p->type_out,
+                             p->variant, p->alpha_re, p->alpha_im, p->beta_re, p->beta_im, false);
+        if (rc != CCGLIB_OK) return rc;
+        p->unfused.store(stand_by, std::memory_order_release);
+      }
     }
-    return ccglib_pipeline_run(p->unfused, d_a, d_b, d_c);
+    return ccglib_pipeline_run(stand_by, d_a, d_b, d_c);
   }
   if (p->int1_direct) {
     ccglib_gemm *g = p->gemm;
