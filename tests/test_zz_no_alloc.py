@@ -3,7 +3,8 @@
 (ccglib_pipeline_create + ccglib_pipeline_run) on the same buffers, two calls in a row, the
 second with a smaller input, so that what the first call left in the array is still there.
 Integer results bit for bit; float results bit for bit where the object takes the same route
-(transposes, then the tiled kernel) and within the float bounds of the oracle elsewhere.
+(transposes, then the tiled kernel) and within the float bounds of the oracle elsewhere; every
+float case is also compared with the oracle itself.
 The device's free memory is read on either side of every stateless call and must not move,
 and the call is captured into a HIP graph and replayed."""
 import numpy as np
@@ -39,18 +40,21 @@ def _inputs(B, M, N, K, tin, axis, seed):
     if tin == VT.int1:
         a = rng.integers(0, 2, B * 2 * M * K, dtype=np.uint8) * rng.integers(1, 256, B * 2 * M * K, dtype=np.uint8)
         b = rng.integers(0, 2, B * 2 * N * K, dtype=np.uint8) * rng.integers(1, 256, B * 2 * N * K, dtype=np.uint8)
-        return a, b      # one byte per sample, in the layout `axis` names
+        return a, b, None, None      # one byte per sample, in the layout `axis` names
     qa = quantize(rng.uniform(-2, 2, (B, 2, M, K)), tin)
     qb = quantize(rng.uniform(-2, 2, (B, 2, N, K)), tin)
+    pa, pb = qa.reshape(-1), qb.reshape(-1)      # planar, as the oracle takes them
     if axis == INTERLEAVED:
         qa = np.ascontiguousarray(qa.transpose(0, 2, 3, 1))
         qb = np.ascontiguousarray(qb.transpose(0, 2, 3, 1))
-    return qa.reshape(-1), qb.reshape(-1)
+    return qa.reshape(-1), qb.reshape(-1), pa, pb
 
 
 def _both(B, M, N, K, tin, tout, axis, c_axis, c_order, variant, alpha, beta, seed):
-    """Runs the object and the stateless call on the same inputs; returns both outputs."""
-    a, b = _inputs(B, M, N, K, tin, axis, seed)
+    """Runs the object and the stateless call on the same inputs; returns both outputs and,
+    for float input, what the oracle says (its float result and the float64 product, both
+    as planar float64 [B][2][rows][cols])."""
+    a, b, pa, pb = _inputs(B, M, N, K, tin, axis, seed)
     rng = np.random.default_rng(seed + 1)
     n_out = B * 2 * M * N
     if tout == VT.int32:
@@ -69,7 +73,22 @@ def _both(B, M, N, K, tin, tout, axis, c_axis, c_order, variant, alpha, beta, se
     free_enqueued = torch.cuda.mem_get_info()[0]
     torch.cuda.synchronize()
     assert free_enqueued == free_before and torch.cuda.mem_get_info()[0] == free_before
-    return to_host(d_c1, OUT_NP[tout]), to_host(d_c2, OUT_NP[tout])
+    oracle = None
+    if pa is not None:
+        order = int(c_order)
+        rows, cols = (M, N) if c_order == ROW else (N, M)
+        c_planar = c_in
+        if c_axis == INTERLEAVED:
+            c_planar = np.ascontiguousarray(c_in.reshape(B, rows, cols, 2).transpose(0, 3, 1, 2)).reshape(-1)
+        want = orc.gemm(pa, pb, M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], order, alpha, beta,
+                        c_planar if complex(beta) != 0 else None)
+        w64 = orc.gemm_float64(pa, pb, M, N, K, ORC_TYPE[tin], order)
+        w = (w64[:, 0] + 1j * w64[:, 1]) * complex(alpha)
+        if complex(beta) != 0:
+            ci = dequantize(c_planar, tout).reshape(w64.shape).astype(np.float64)
+            w = w + complex(beta) * (ci[:, 0] + 1j * ci[:, 1])
+        oracle = (dequantize(want, tout).astype(np.float64), np.stack([w.real, w.imag], axis=1))
+    return to_host(d_c1, OUT_NP[tout]), to_host(d_c2, OUT_NP[tout]), oracle
 
 
 # (first call, second and smaller call) per case
@@ -100,8 +119,8 @@ def test_static_pipeline_matches_pipeline_object(case):
     for n, (B, M, N, K) in enumerate(case["shapes"]):
         print("static pipeline call %d: B=%d M=%d N=%d K=%d %s" % (n, B, M, N, K, case["tin"].name), flush=True)
         tin, tout = case["tin"], case["tout"]
-        obj, static = _both(B, M, N, K, tin, tout, case["axis"], case["c_axis"], case["c_order"],
-                            case["variant"], case["alpha"], case["beta"], seed=17 + n)
+        obj, static, oracle = _both(B, M, N, K, tin, tout, case["axis"], case["c_axis"], case["c_order"],
+                                    case["variant"], case["alpha"], case["beta"], seed=17 + n)
         if case["exact"]:
             assert np.array_equal(obj, static)
         else:
@@ -109,6 +128,13 @@ def test_static_pipeline_matches_pipeline_object(case):
             # for the oracle's float product and float64 product
             o = dequantize(obj, tout).astype(np.float64)
             check_float(dequantize(static, tout), o, o, tin, tout)
+        if oracle is not None:
+            # and against the oracle itself (planar view of what the call wrote)
+            rows, cols = (M, N) if case["c_order"] == ROW else (N, M)
+            got = dequantize(static, tout)
+            got = (got.reshape(B, rows, cols, 2).transpose(0, 3, 1, 2) if case["c_axis"] == INTERLEAVED
+                   else got.reshape(B, 2, rows, cols))
+            check_float(np.ascontiguousarray(got), oracle[0], oracle[1], tin, tout)
 
 
 def test_static_pipeline_against_oracle():
