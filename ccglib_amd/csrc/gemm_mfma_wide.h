@@ -1,7 +1,8 @@
 // Wide-block variant of the direct-to-LDS complex GEMM for 16-bit input in the
-// tiled (opt) layout: a 192 x 256 patch of C per block, four waves (one per SIMD,
-// the whole register file each) of 192 x 64, i.e. 12 x 4 MFMA tiles of 16 x 16 and
-// 384 accumulator registers per lane.
+// tiled (opt) layout - or, as a second instantiation, in the caller's rows of
+// (re, im) pairs, see IL below: a 192 x 256 patch of C per block, four waves (one
+// per SIMD, the whole register file each) of 192 x 64, i.e. 12 x 4 MFMA tiles of
+// 16 x 16 and 384 accumulator registers per lane.
 //
 // Compared with the 256 x 128 block of complex_gemm_mfma_dtl this moves 22 % fewer
 // bytes from L2 to LDS per flop (448 operand rows per 49152 products instead of
