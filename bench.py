@@ -126,8 +126,44 @@ def check_result(name, a, b, c, torch):
             "batch": bi}
 
 
+def sample_core_clock(run, torch, load_s=1.2):
+    """The core clock while `run` is enqueued over and over: rocm-smi is asked once, from a
+    thread, about a third into `load_s` seconds of load. Returns MHz, or None when rocm-smi
+    is not there or says nothing that parses (the figure is reported, not relied on)."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    tool = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    if not os.path.exists(tool):
+        return None
+    found = []
+
+    def ask():
+        time.sleep(load_s / 3)
+        try:
+            out = subprocess.run([tool, "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+            m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
+            if m:
+                found.append(float(m.group(1)))
+        except Exception:
+            pass
+
+    t = threading.Thread(target=ask)
+    t.start()
+    t0 = time.perf_counter()
+    while t.is_alive() or time.perf_counter() - t0 < load_s:
+        for _ in range(16):
+            run()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 > 30:
+            break
+    t.join()
+    return found[0] if found else None
+
+
 def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_calibration=False,
-            check=True):
+            check=True, clock=False):
     """Builds the step of a workload, settles, times `steps` steps and checks the result.
     Returns a dict of figures plus what the optional extra measurements need."""
     stream = torch.cuda.current_stream().cuda_stream
@@ -312,6 +348,9 @@ def measure(name, steps, warmup, settle_ms, torch, np, cc, isolated=False, copy_
         torch.cuda.synchronize()
         iso_ms = e0.elapsed_time(e1) / iters
         out["isolated"] = {"gemm_ms": iso_ms, "gemm_tflops": flops / (iso_ms * 1e-3) / 1e12}
+    if clock:
+        # core clock under this workload's steps, after everything that is timed
+        out["sclk_mhz"] = sample_core_clock(step, torch)
     out["_buffers"] = (a_in, b_in, c)    # for the optional pipeline measurements of the caller
     return out
 
@@ -332,6 +371,8 @@ def main():
                          "in `other_workloads` (0: skip them)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-clock", action="store_true",
+                    help="do not sample the core clock under load with rocm-smi after the timed steps")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 1 GiB device copy (for scaling rocprofv3 HBM counters)")
     ap.add_argument("--isolated", action="store_true",
@@ -359,7 +400,7 @@ def main():
     tin, tout = VT[tin_name], VT[tout_name]
     m = measure(name, args.steps, args.warmup, args.settle_ms, torch, np, cc,
                 isolated=args.isolated, copy_calibration=args.copy_calibration,
-                check=not args.no_check)
+                check=not args.no_check, clock=not args.no_clock)
     a_in, b_in, c = m.pop("_buffers")
     flops, value, ms_per_step = m["flops"], m["value"], m["ms_per_step"]
     gemm_ms, gemm_tflops, peak = m["gemm_ms"], m["gemm_tflops"], m["peak"]
@@ -386,6 +427,13 @@ def main():
                      "traffic": traffic, "traffic_source": traffic_source, "kernel_ms": gemm_ms},
         "kernels": m["per_kernel"],
     }
+    if m.get("sclk_mhz"):
+        # The published peak is CUs x flop per clock and CU x 2.4 GHz; at the clock the part
+        # actually runs under this load (power limit) the same formula gives a lower roof.
+        sclk = m["sclk_mhz"]
+        result["roofline"]["sclk_mhz_under_load"] = sclk
+        result["roofline"]["peak_at_measured_clock"] = peak * sclk / 2400.0
+        result["roofline"]["frac_of_peak_at_measured_clock"] = gemm_tflops / (peak * sclk / 2400.0)
     result.update(m["info"])
     if "isolated" in m:
         result["isolated"] = m["isolated"]
@@ -471,7 +519,7 @@ def main():
         others = {}
         for other in ("square_bf16", "square_bf16_out", "fp8_e4m3", "fp8_e5m2", "correlator_int1"):
             o = measure(other, args.other_steps, 3, args.settle_ms, torch, np, cc,
-                        check=not args.no_check)
+                        check=not args.no_check, clock=not args.no_clock)
             o.pop("_buffers")
             others[other] = {
                 "kernel": o["kernel_name"], "shape": dict(zip("BMNK", o["shape"])),
@@ -480,6 +528,10 @@ def main():
                 "unit": o["unit"], "frac": o["gemm_tflops"] / o["peak"],
                 "ms_per_step": o["ms_per_step"], "step_rate": o["value"],
                 "kernels": o["per_kernel"], "check": o["check"]}
+            if o.get("sclk_mhz"):
+                others[other]["sclk_mhz_under_load"] = o["sclk_mhz"]
+                others[other]["frac_of_peak_at_measured_clock"] = \
+                    o["gemm_tflops"] / (o["peak"] * o["sclk_mhz"] / 2400.0)
             del o
             torch.cuda.empty_cache()
         result["other_workloads"] = others
