@@ -52,13 +52,45 @@ def _compile(src, force):
     path = os.path.join(CSRC, src)
     if not force and not _stale(obj, [path] + HEADERS):
         return obj, ""
-    cmd = [_hipcc()] + HIPCC_FLAGS + _defines() + ["-c", path, "-o", obj]
+    cmd = [_hipcc()] + HIPCC_FLAGS + _defines() + ["-Rpass-analysis=kernel-resource-usage", "-c", path,
+                                                   "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
-                    if "packed-fp32-ops" not in l)
+    lines = (r.stdout + r.stderr).splitlines()
+    kept, skip = [], 0
+    for l in lines:      # (the remarks, each with its source line and caret, stay out of the log)
+        if "kernel-resource-usage" in l:
+            skip = 2
+        elif skip and (l.lstrip()[:1].isdigit() or l.strip().startswith("|")):
+            skip -= 1
+        elif "packed-fp32-ops" not in l:
+            kept.append(l)
+            skip = 0
+    log = "\n".join(kept)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    _no_scratch_in_gemm_kernels(src, lines)
     return obj, log
+
+
+def _no_scratch_in_gemm_kernels(src, remarks):
+    """The MFMA GEMM kernels wait for their copies with explicit `s_waitcnt vmcnt(n)` counts,
+    which only hold while the compiler adds no memory instructions of its own inside the K
+    loop. The compiler's resource remarks say whether a kernel spills registers to scratch
+    memory. The one-wave-per-SIMD kernels (complex_gemm_mfma_wide) run at the edge of the
+    register file and must not spill at all: the build stops if one does. Of the others, the
+    1-bit 128 x 128 kernel spills four values at set-up and reloads them where a block moves
+    to its next C tile (the compiler waits for all memory operations there); anything beyond
+    those few bytes stops the build as well."""
+    name = None
+    for l in remarks:
+        if "Function Name:" in l:
+            name = l.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in l and name and "complex_gemm_mfma" in name:
+            size = int(l.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if size > (0 if "complex_gemm_mfma_wide" in name else 32):
+                os.remove(os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o"))
+                raise RuntimeError("%s: kernel %s spills %d bytes per lane to scratch memory; its "
+                                   "explicit vmcnt counts would not hold" % (src, name, size))
 
 
 def build(force=False, verbose=False):

@@ -821,7 +821,7 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
   // with the break-even T of large problems and c the launches' fixed cost in
   // operand elements. Measured (python -m ccglib_amd.tuning.pipeline_crossover at
   // K = 256, 1024, 4096): 16-bit interleaved rows T = 3800 where the 192 x 256 kernel
-  // reads them (planar C, no alpha / beta, M and N multiples of 64, K of 32) and
+  // reads them (planar C, no beta, alpha only with fp32 C, M and N multiples of 64, K of 32) and
   // 2800 elsewhere, 8-bit interleaved rows T = 2700, c = 1e7 for both.
   const double mn_over_sum = (M + N) ? (double)M * (double)N / (double)(M + N) : 0.0;
   const double operand_elements = (double)B * (double)K * (double)(M + N);
@@ -832,8 +832,9 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
            (route == 0 && operand_elements > 0 &&
             mn_over_sum < break_even * (1.0 + fixed_cost / operand_elements));
   };
+  const bool no_alpha = alpha_re == 1.f && alpha_im == 0.f;
   const bool wide_rows = in_bits == 16 && output_complex_axis_location == kPlanar &&
-                         alpha_re == 1.f && alpha_im == 0.f && beta_re == 0.f && beta_im == 0.f &&
+                         beta_re == 0.f && beta_im == 0.f && (no_alpha || output_type == kFloat32) &&
                          M % 64 == 0 && N % 64 == 0 && K % 32 == 0 && K >= 64;
   const bool fused = allow_fused && !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&

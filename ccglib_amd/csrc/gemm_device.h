@@ -107,6 +107,15 @@ struct KernelArgs {
   unsigned im_excess;
 };
 
+// alpha * (re + i im), one part at a time. The fused operation is written out, so that
+// every kernel that applies alpha rounds alike whatever the compiler would contract.
+__device__ __forceinline__ float alpha_times_re(float ar, float ai, float re, float im) {
+  return __builtin_fmaf(ar, re, -(ai * im));
+}
+__device__ __forceinline__ float alpha_times_im(float ar, float ai, float re, float im) {
+  return __builtin_fmaf(ai, re, ar * im);
+}
+
 // Maps the hardware workgroup id to a logical tile id such that the ids that
 // one XCD receives (every 8th workgroup) are consecutive.
 __device__ __forceinline__ unsigned xcd_remap(unsigned wg, unsigned total) {

@@ -887,8 +887,8 @@ __device__ __forceinline__ void store_wave_tile(const KernelArgs &args, unsigned
         im[e] = piece_elem<MS, TILE0>(acc_im, j, i, e);
         if (have_alpha) {
           const float r0 = re[e];
-          re[e] = ar * r0 - ai * im[e];
-          im[e] = ai * r0 + ar * im[e];
+          re[e] = alpha_times_re(ar, ai, r0, im[e]);
+          im[e] = alpha_times_im(ar, ai, r0, im[e]);
         }
       }
       const bool full = vec_ok && (x + 4 <= nx);
@@ -1084,8 +1084,8 @@ __device__ __forceinline__ void store_wave_tile_rows(const KernelArgs &args, uns
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float re = acc_re[j][i][e], im = acc_im[j][i][e];
-          v[i] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
-                            : (have_alpha ? ai * re + ar * im : im);
+          v[i] = plane == 0 ? (have_alpha ? alpha_times_re(ar, ai, re, im) : re)
+                            : (have_alpha ? alpha_times_im(ar, ai, re, im) : im);
         }
         Tout *p = out + (size_t)plane * nx * ny + (size_t)(j * 16 + e) * nx;
         if constexpr (kAblateStores) {
@@ -1132,8 +1132,8 @@ __device__ __forceinline__ void store_wave_tile_staged(const KernelArgs &args, u
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float re = acc_re[j][i][e], im = acc_im[j][i][e];
-          v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
-                            : (have_alpha ? ai * re + ar * im : im);
+          v[e] = plane == 0 ? (have_alpha ? alpha_times_re(ar, ai, re, im) : re)
+                            : (have_alpha ? alpha_times_im(ar, ai, re, im) : im);
         }
         *reinterpret_cast<float4_t *>(wr + i * 64) = v;
       }
@@ -1175,8 +1175,8 @@ __device__ __forceinline__ void store_wave_tile_staged_narrow(const KernelArgs &
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float re = acc_re[j][i][e], im = acc_im[j][i][e];
-          v[e] = (Tout)(plane == 0 ? (have_alpha ? ar * re - ai * im : re)
-                                   : (have_alpha ? ai * re + ar * im : im));
+          v[e] = (Tout)(plane == 0 ? (have_alpha ? alpha_times_re(ar, ai, re, im) : re)
+                                   : (have_alpha ? alpha_times_im(ar, ai, re, im) : im));
         }
         *reinterpret_cast<ushort4_t *>(wr + i * 32) = __builtin_bit_cast(ushort4_t, v);
       }
@@ -1214,8 +1214,8 @@ __device__ __forceinline__ void store_wave_tile_staged_il(const KernelArgs &args
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float r0 = acc_re[j][i][e], i0 = acc_im[j][i][e];
-          re[e] = have_alpha ? ar * r0 - ai * i0 : r0;
-          im[e] = have_alpha ? ai * r0 + ar * i0 : i0;
+          re[e] = have_alpha ? alpha_times_re(ar, ai, r0, i0) : r0;
+          im[e] = have_alpha ? alpha_times_im(ar, ai, r0, i0) : i0;
         }
         char *w = wr + (i - 2 * h) * 128;
         *reinterpret_cast<float4_t *>(w) = float4_t{re[0], im[0], re[1], im[1]};
@@ -1266,8 +1266,8 @@ __device__ __forceinline__ void store_wave_tile_staged32(const KernelArgs &args,
               const unsigned o = plane == 0 ? iar * sr - iai * si : iai * sr + iar * si;
               v[e] = __builtin_bit_cast(float, o);
             } else {
-              v[e] = plane == 0 ? (have_alpha ? ar * re - ai * im : re)
-                                : (have_alpha ? ai * re + ar * im : im);
+              v[e] = plane == 0 ? (have_alpha ? alpha_times_re(ar, ai, re, im) : re)
+                                : (have_alpha ? alpha_times_im(ar, ai, re, im) : im);
             }
           }
           *reinterpret_cast<float4_t *>(wr + k * 32) = v;
@@ -1439,6 +1439,13 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
 // Both copy helpers write m0 (the LDS base of the copy) and say so in their
 // clobber lists, so that the compiler never assumes a value it put there
 // survives them; clang warns about any mention of m0 there, which is the point.
+// The compiler does not look into an asm statement for the wait states its
+// instructions need after what it placed in front of it: the scalar base of the
+// first helper may have come out of a vector register shortly before (a spilled
+// scalar register read back with v_readlane), and a vector memory instruction
+// may read such a register five wait states later at the earliest. In the code
+// as generated the address arithmetic between the two is longer than that;
+// tests/test_kernel_asm.py checks it.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_offset,
@@ -1992,12 +1999,25 @@ hipError_t launch_wide(const GemmParams &p, hipStream_t stream) {
   const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL>;
-  static std::atomic<bool> lds_allowed[kMaxDevices];
-  if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
   const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
   const unsigned grid = (unsigned)(total < resident ? total : resident);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
+  if (p.have_alpha) {
+    // (interleaved rows, alpha and a 16-bit C together need more registers than a
+    // lane has; wide_tiles_apply keeps that combination away)
+    if constexpr (IL && TOUT != kFloat32) {
+      return hipErrorInvalidValue;
+    } else {
+      auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL, true>;
+      static std::atomic<bool> lds_allowed[kMaxDevices];
+      if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
+    }
+  } else {
+    auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL, false>;
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
+  }
   return hipGetLastError();
 }
 
@@ -2024,11 +2044,12 @@ inline bool small_tiles_pay(const GemmParams &p, double penalty) {
 // outside C), but its tiles are 1.5 times as large, so more of the last round of
 // tiles can stay empty (8192^3: 5.4 rounds of 192 x 256 tiles against 8 full ones).
 inline bool wide_tiles_apply(const GemmParams &p) {
-  if (p.c_interleaved || p.have_alpha || p.have_beta || (uintptr_t)p.c % 16 != 0 ||
+  if (p.c_interleaved || p.have_beta || (uintptr_t)p.c % 16 != 0 ||
       p.nx % 64 != 0 || p.ny % 64 != 0 || p.k_in_memory) {
     return false;
   }
   if (p.input_interleaved) {
+    if (p.have_alpha && p.type_out != kFloat32) return false;   // (registers, see launch_wide)
     // rows of whole 128-byte pieces (32 complex values), at least two of them; a
     // lane's offset inside a copy of 8 rows is a 32-bit number
     const size_t row_bytes = (size_t)2 * p.k * bits_of(p.type_in) / 8;
@@ -2081,8 +2102,8 @@ hipError_t launch_typed(const GemmParams &p, hipStream_t stream) {
   }
   if (p.variant == kOpt || planar_direct) {
     if constexpr (KPM == 1 && DtypeTraits<DT>::kElemBytes == 2) {
-      // 16-bit input, tiled operands, planar C with neither alpha nor beta: 192 x 256
-      // block, 4 waves of 192 x 64 (one per SIMD), where that pays
+      // 16-bit input, tiled operands, planar C without beta: 192 x 256 block, 4 waves
+      // of 192 x 64 (one per SIMD), where that pays
       if (wide_tiles_apply(p) && wide_tiles_pay(p)) return launch_wide<DT, TOUT>(p, stream);
     }
     if constexpr (KPM == 1) {

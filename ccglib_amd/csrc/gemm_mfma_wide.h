@@ -53,9 +53,15 @@ constexpr int kWideTX = kWideBX / 16;   // X tiles of a wave
 // as AccVGPRs (all 256) and those of the last four as ordinary VGPRs, and stay
 // where they are. What the compiler no longer does for these statements: the
 // wait states between a matrix instruction and a dependent read of its result by
-// another kind of instruction; the epilogue waits explicitly
-// (wait_for_mfma_results). A matrix instruction that adds to the result of the
-// one before needs none.
+// another kind of instruction - the epilogue waits explicitly
+// (wait_for_mfma_results) - and the wait states between a vector-ALU write of an
+// operand register and the matrix instruction that reads it: every value derived
+// from a fragment is therefore pinned several matrix instructions ahead of its
+// use (flip_sign, swap_pairs), and tests/test_kernel_asm.py scans the generated
+// code for a vector-ALU write right in front of a matrix instruction that reads
+// it. (An s_nop in front of every matrix instruction would do as well and
+// measured 6 % slower.) A matrix instruction that adds to the result of the one
+// before needs none.
 // ZERO: the sum starts from zero (first K tile of a C tile).
 template <int DT, bool ACC_IN_AGPR, bool ZERO>
 __device__ __forceinline__ void mfma16_asm(float4_t &acc, const int4_t &a, const int4_t &b) {
@@ -142,7 +148,9 @@ __device__ __forceinline__ TileCoord tile_coord_by_lane(const KernelArgs &args, 
 // instruction fetches 8 whole 128-byte lines, and every fragment read touches
 // the banks exactly as in the tiled layout (64-byte rows, 256 bytes apart every
 // four), so the chunk swizzles of that layout carry over.
-template <int DT, int TOUT, bool IL>
+// ALPHA: the result is multiplied by the complex alpha of the arguments on its way
+// out (both parts of an element sit in the same lane, in acc_re and acc_im).
+template <int DT, int TOUT, bool IL, bool ALPHA>
 __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArgs args) {
   static_assert(DtypeTraits<DT>::kTilesPerMfma == 1 && DtypeTraits<DT>::kElemBytes == 2,
                 "16-bit input");
@@ -411,7 +419,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   //   group 1 (tiles 4 - 7): half in the last iteration, half in the next first one
   //   (which starts these accumulators again with its tile 4);
   //   group 2 (tiles 8 - 11): the next first iteration, before its tile 8.
-  // The host only launches this kernel for planar C without alpha and beta, with
+  // The host only launches this kernel for planar C without beta, with
   // 16-byte aligned rows and nx, ny multiples of 64: a 64 x 64 piece of a tile is
   // either inside C or outside.
   using Tout = typename OutType<TOUT>::type;
@@ -443,14 +451,36 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   auto store_piece = [&](int g, int s) {
     if (!target.inside[g]) return;
     const int j = s >> 3, plane = (s >> 2) & 1, e = s & 3;
-    float4_t(&acc)[4][TX] = plane == 0 ? acc_re : acc_im;
-    if (g < 2) {
-      take_accumulators<true>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+    float v[4];
+    if constexpr (ALPHA) {
+      // both parts of the four elements; the expressions of the other kernels'
+      // epilogues, so that the compiler contracts them alike and every block tile
+      // gives the same bits
+      if (g < 2) {
+        take_accumulators<true>(acc_re[j][4 * g], acc_re[j][4 * g + 1], acc_re[j][4 * g + 2], acc_re[j][4 * g + 3]);
+        take_accumulators<true>(acc_im[j][4 * g], acc_im[j][4 * g + 1], acc_im[j][4 * g + 2], acc_im[j][4 * g + 3]);
+      } else {
+        take_accumulators<false>(acc_re[j][4 * g], acc_re[j][4 * g + 1], acc_re[j][4 * g + 2], acc_re[j][4 * g + 3]);
+        take_accumulators<false>(acc_im[j][4 * g], acc_im[j][4 * g + 1], acc_im[j][4 * g + 2], acc_im[j][4 * g + 3]);
+      }
+      const float ar = args.alpha_re, ai = args.alpha_im;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float re = acc_re[j][4 * g + i][e], im = acc_im[j][4 * g + i][e];
+        v[i] = plane == 0 ? alpha_times_re(ar, ai, re, im) : alpha_times_im(ar, ai, re, im);
+      }
     } else {
-      take_accumulators<false>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+      float4_t(&acc)[4][TX] = plane == 0 ? acc_re : acc_im;
+      if (g < 2) {
+        take_accumulators<true>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+      } else {
+        take_accumulators<false>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+      }
+      v[0] = acc[j][4 * g][e];
+      v[1] = acc[j][4 * g + 1][e];
+      v[2] = acc[j][4 * g + 2][e];
+      v[3] = acc[j][4 * g + 3][e];
     }
-    const float v[4] = {acc[j][4 * g][e], acc[j][4 * g + 1][e], acc[j][4 * g + 2][e],
-                        acc[j][4 * g + 3][e]};
     char *p = target.base + plane * plane_bytes +
               ((size_t)(j * 16 + e) * args.nx + g * 64) * sizeof(Tout) + lane_store_off;
     if constexpr (kAblateStores) {

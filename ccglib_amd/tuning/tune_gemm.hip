@@ -87,9 +87,9 @@ static const std::vector<Config> kConfigs = {
     {"f16 256x128 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 y3 x4 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true, 4>, kFloat16, kFloat32},
-    {"f16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32>, kFloat16, kFloat32},
+    {"f16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32, false>, kFloat16, kFloat32},
     {"bf16 256x128 w64x64 s3 m16 xt", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kBfloat16, kFloat32},
-    {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32>, kBfloat16, kFloat32},
+    {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32, false>, kBfloat16, kFloat32},
 #ifndef TUNE_GEMM_SMALL
     {"f16 256x128 w64x64 s3 m32", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 32>, kFloat16, kFloat32},
     {"f16 128x128 w64x64 s2 m16", launch_dtl<kFloat16, kFloat32, 128, 128, 64, 64, 2, 2, kLoadTiled, 16>, kFloat16, kFloat32},
@@ -482,7 +482,7 @@ int main(int argc, char **argv) {
     p.beta_im = 0;
     p.have_alpha = 0;
     p.have_beta = 0;
-    if (c.launch == launch_wide<kFloat16, kFloat32> || c.launch == launch_wide<kBfloat16, kFloat32> ||
+    if (c.launch == launch_wide<kFloat16, kFloat32, false> || c.launch == launch_wide<kBfloat16, kFloat32, false> ||
         c.launch == launch_wide<kFloat16, kFloat32, true> ||
         c.launch == launch_wide<kBfloat16, kFloat32, true>) {
       if (!wide_tiles_apply(p)) {

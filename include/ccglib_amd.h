@@ -88,7 +88,7 @@ CCGLIB_API const char *ccglib_version(void);
  *                    operands use 256 x 128 block tiles, 128 x 128 ones when
  *                    the larger would leave compute units idle (small
  *                    problems), or 192 x 256 ones (16-bit tiled input, planar C
- *                    without alpha or beta, M and N multiples of 64, K of more
+ *                    without beta, M and N multiples of 64, K of more
  *                    than 32) when those fill the compute units well enough;
  *                    1: always 256 x 128; 2: always 128 x 128; 3: 192 x 256
  *                    wherever that kernel applies, else as 0. The 192 x 256

@@ -525,7 +525,7 @@ def test_block_tiles_int1(block_tile, variant):
 @pytest.mark.parametrize("c_order", [ROW, COL])
 def test_wide_block_tile(tin, tout, c_order):
     """GEMM_BLOCK_TILE = 3: the 192 x 256 block (16-bit tiled input, planar C without
-    alpha or beta, M and N multiples of 64, K of more than one tile) against the
+    beta, M and N multiples of 64, K of more than one tile) against the
     oracle: tiles that lie inside C and tiles of which only one or two 64-column
     groups or some of the four 64-row pieces do, two to many K tiles, more C tiles
     than compute units, and a K with a partial last tile."""
@@ -535,15 +535,19 @@ def test_wide_block_tile(tin, tout, c_order):
         float_case(1, 64, 64, 40, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=3)
         float_case(2, 512, 832, 1000, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=4)
         float_case(40, 256, 576, 72, tin, tout, cc.Variant.opt, PLANAR, c_order, signed=False, seed=5)
+        # with a complex alpha (applied to the accumulators on their way out)
+        float_case(3, 320, 448, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=1.5 - 0.5j, seed=6)
+        float_case(2, 256, 192, 2048, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=-0.25 + 2j, seed=7)
 
 
 def test_wide_block_tile_falls_back():
     """GEMM_BLOCK_TILE = 3 where the 192 x 256 kernel does not apply (ragged M or N,
-    alpha / beta, interleaved C, K of one tile, fp8): the other kernels compute it."""
+    beta, interleaved C, K of one tile, fp8): the other kernels compute it."""
     with cc.option(cc.Option.gemm_block_tile, 3):
         float_case(2, 300, 520, 96, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=1)
         float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW,
                    alpha=1.5 - 0.5j, beta=0.25 + 1j, seed=2)
+        float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW, beta=1, seed=7)
         float_case(1, 256, 192, 64, VT.float16, VT.float32, cc.Variant.opt, INTERLEAVED, ROW, seed=3)
         float_case(1, 256, 192, 32, VT.float16, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=4)
         float_case(1, 256, 192, 128, VT.float8e4m3, VT.float32, cc.Variant.opt, PLANAR, ROW, seed=5)
@@ -551,16 +555,17 @@ def test_wide_block_tile_falls_back():
 
 
 @pytest.mark.parametrize("B,M,N,K", [(2, 384, 640, 256), (3, 512, 4096, 576), (1, 1024, 1216, 2048)])
-def test_block_tile_choice_is_invisible(B, M, N, K):
+@pytest.mark.parametrize("alpha", [1, 0.75 - 1.25j])
+def test_block_tile_choice_is_invisible(B, M, N, K, alpha):
     """The same bits whichever block tile computes them (same K order per element, and
-    per K tile the same order of the four real products)."""
+    per K tile the same order of the four real products; the same expression for alpha)."""
     rng = np.random.default_rng(11)
     qa = quantize(rng.standard_normal((B, 2, M, K)).astype(np.float32), VT.float16).reshape(-1)
     qb = quantize(rng.standard_normal((B, 2, N, K)).astype(np.float32), VT.float16).reshape(-1)
     results = []
     for block_tile in (0, 1, 2, 3):
         with cc.option(cc.Option.gemm_block_tile, block_tile):
-            results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt))
+            results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt, alpha=alpha))
     for r in results[1:]:
         assert np.array_equal(results[0], r)
 

@@ -472,12 +472,13 @@ def test_pipeline_planar_rows_read_in_place(tin, K, skew):
 @pytest.mark.parametrize("c_order", [ROW, COL])
 def test_pipeline_interleaved_rows_wide_block(tin, tout, c_order):
     """GEMM_BLOCK_TILE = 3 for 16-bit interleaved rows read in place: the 192 x 256 block
-    (planar C without alpha or beta, M and N multiples of 64, rows of whole 128-byte
+    (planar C without beta, M and N multiples of 64, rows of whole 128-byte
     pieces, i.e. K a multiple of 32) against the oracle, and bit for bit against the
     256 x 128 block: tiles inside C and tiles of which only some 64-column groups or
     64-row pieces are, two to many K pieces, more C tiles than compute units."""
-    for seed, (B, M, N, K) in enumerate([(2, 256, 192, 64), (3, 320, 448, 96), (2, 512, 832, 992),
-                                         (40, 256, 576, 64), (1, 64, 64, 128)]):
+    for seed, (B, M, N, K, alpha) in enumerate([(2, 256, 192, 64, 1), (3, 320, 448, 96, 1),
+                                                (2, 512, 832, 992, 1), (40, 256, 576, 64, 1),
+                                                (1, 64, 64, 128, 1), (3, 320, 448, 96, 0.5 - 1.5j)]):
         rng = np.random.default_rng(40 + seed)
         qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), tin)
         qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), tin)
@@ -488,13 +489,16 @@ def test_pipeline_interleaved_rows_wide_block(tin, tout, c_order):
         for block_tile in (3, 1):
             with cc.option(cc.Option.gemm_block_tile, block_tile):
                 p = cc.Pipeline(B, M, N, K, 0, stream(), INTERLEAVED, PLANAR, ROW, COL, c_order, tin, tout,
-                                cc.Variant.opt)
+                                cc.Variant.opt, alpha)
             d_c = to_device(np.full(B * 2 * M * N, np.nan, dtype=np.float32) if tout == VT.float32
                             else np.full(B * 2 * M * N, 0x7fc0, dtype=np.uint16))
             p.Run(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr())
             torch.cuda.synchronize()
             results.append(to_host(d_c, out_np))
-        want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], int(c_order))
+        want = orc.gemm(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], ORC_TYPE[tout], int(c_order),
+                        alpha)
         w64 = orc.gemm_float64(qa.reshape(-1), qb.reshape(-1), M, N, K, ORC_TYPE[tin], int(c_order))
+        w = (w64[:, 0] + 1j * w64[:, 1]) * complex(alpha)
+        w64 = np.stack([w.real, w.imag], axis=1)
         check_float(dequantize(results[0], tout).reshape(want.shape), dequantize(want, tout), w64, tin, tout)
         assert np.array_equal(results[0], results[1]), (B, M, N, K)
