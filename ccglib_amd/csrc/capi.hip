@@ -832,9 +832,8 @@ int pipeline_create(ccglib_pipeline_t *pipeline, size_t B, size_t M, size_t N, s
            (route == 0 && operand_elements > 0 &&
             mn_over_sum < break_even * (1.0 + fixed_cost / operand_elements));
   };
-  const bool no_alpha = alpha_re == 1.f && alpha_im == 0.f;
   const bool wide_rows = in_bits == 16 && output_complex_axis_location == kPlanar &&
-                         beta_re == 0.f && beta_im == 0.f && (no_alpha || output_type == kFloat32) &&
+                         beta_re == 0.f && beta_im == 0.f &&
                          M % 64 == 0 && N % 64 == 0 && K % 32 == 0 && K >= 64;
   const bool fused = allow_fused && !packing && input_complex_axis_location == kInterleaved && K > 0 &&
                      (in_bits == 8 || in_bits == 16) && (2 * K * in_bits / 8) % 16 == 0 &&

@@ -99,6 +99,8 @@ struct KernelArgs {
   // in memory, of which this launch may cover a piece of K
   unsigned row_stride_bytes, k_tile_stride;
   unsigned blocks_x, blocks_y;
+  // 192 x 256 kernel only: tiles of 128 columns that follow the blocks_x full ones of a row
+  unsigned short_x;
   size_t x_batch_bytes, y_batch_bytes;
   float alpha_re, alpha_im, beta_re, beta_im;
   int have_alpha, have_beta, c_interleaved;
@@ -108,12 +110,20 @@ struct KernelArgs {
 };
 
 // alpha * (re + i im), one part at a time. The fused operation is written out, so that
-// every kernel that applies alpha rounds alike whatever the compiler would contract.
+// every kernel that applies alpha rounds alike whatever the compiler would contract,
+// and the float result is taken by an empty asm statement: a conversion to fp16 that
+// follows is then a rounding of that float (as in the reference, which stores the
+// float sum into a half) and cannot be merged into the fused operation, which would
+// round the exact sum once.
 __device__ __forceinline__ float alpha_times_re(float ar, float ai, float re, float im) {
-  return __builtin_fmaf(ar, re, -(ai * im));
+  float r = __builtin_fmaf(ar, re, -(ai * im));
+  asm("" : "+v"(r));
+  return r;
 }
 __device__ __forceinline__ float alpha_times_im(float ar, float ai, float re, float im) {
-  return __builtin_fmaf(ai, re, ar * im);
+  float r = __builtin_fmaf(ai, re, ar * im);
+  asm("" : "+v"(r));
+  return r;
 }
 
 // Maps the hardware workgroup id to a logical tile id such that the ids that
@@ -219,6 +229,7 @@ inline KernelArgs make_kernel_args(const GemmParams &p, int bx, int by) {
   a.k_tile_stride = p.k_in_memory ? (unsigned)ceil_div(k_mem, (size_t)k_per_tile(p.type_in)) : p.k_tiles;
   a.blocks_x = (unsigned)ceil_div(p.nx, bx);
   a.blocks_y = (unsigned)ceil_div(p.ny, by);
+  a.short_x = 0;
   if (p.variant == kOpt && !p.input_interleaved) {
     a.x_batch_bytes = (size_t)p.x_tiles * a.k_tile_stride * kTileBytes;
     a.y_batch_bytes = (size_t)p.y_tiles * a.k_tile_stride * kTileBytes;

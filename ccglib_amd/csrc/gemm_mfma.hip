@@ -29,6 +29,7 @@
 //    XCD (shared L2), in groups that reuse both operands.
 #include <atomic>
 #include <type_traits>
+#include <utility>
 
 #include "gemm_device.h"
 
@@ -1441,21 +1442,23 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_then_barrier() {
 // survives them; clang warns about any mention of m0 there, which is the point.
 // The compiler does not look into an asm statement for the wait states its
 // instructions need after what it placed in front of it: the scalar base of the
-// first helper may have come out of a vector register shortly before (a spilled
+// first helper may have come out of a vector register right before (a spilled
 // scalar register read back with v_readlane), and a vector memory instruction
-// may read such a register five wait states later at the earliest. In the code
-// as generated the address arithmetic between the two is longer than that;
-// tests/test_kernel_asm.py checks it.
+// may read such a register five wait states later at the earliest. The helper
+// therefore hands the base on through a scalar move: the scalar ALU may read the
+// register at once, and what it writes the memory instruction may read at once.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_1k_to_lds(const char *base, unsigned lane_offset,
                                                unsigned lds_address) {
   if constexpr (kAblateCopies) return;
+  unsigned long long base_here;
   asm volatile(
-      "s_mov_b32 m0, %0\n\t"
+      "s_mov_b64 %0, %3\n\t"
+      "s_mov_b32 m0, %1\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
-      :
+      "global_load_lds_dwordx4 %2, %0"
+      : "=&s"(base_here)
       : "s"(lds_address), "v"(lane_offset), "s"(base)
       : "memory", "m0");
 }
@@ -1991,27 +1994,68 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// How the 192 x 256 kernel covers the width of C: tiles of 192 columns, the last of
+// which may hang over the edge, or - where 64 divides the width - full tiles
+// followed by one or two of 128 columns (4096 = 20 x 192 + 2 x 128), which take two
+// thirds of the matrix instructions. The short tiles are the last ones in the
+// kernel's numbering, and a block computes its full tiles before its short ones;
+// `rounds` is the work of the block that finishes last, in full tiles (B=64
+// 512x4096: 10 2/3 instead of 11), with a charge for the change of kind.
+struct WideTiling {
+  unsigned full_x, short_x, grid;
+  double rounds;
+};
+// (the tuner switches the short tiles off for a row of its table)
+static bool g_wide_short_tiles = true;
+inline WideTiling wide_tiling(const GemmParams &p) {
+  const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
+  const size_t rows = ceil_div((size_t)p.ny, (size_t)kWideBY) * p.batch;
+  WideTiling plain;
+  plain.full_x = (unsigned)ceil_div((size_t)p.nx, (size_t)kWideBX);
+  plain.short_x = 0;
+  const size_t plain_total = plain.full_x * rows;
+  plain.grid = (unsigned)(plain_total < resident ? plain_total : resident);
+  plain.rounds = plain.grid ? (double)ceil_div(plain_total, (size_t)plain.grid) : 0.0;
+  const size_t units = p.nx / 64;
+  const unsigned n_short = units % 3 == 0 ? 0 : units % 3 == 2 ? 1 : 2;
+  if (!g_wide_short_tiles || p.nx % 64 != 0 || n_short == 0 || units < 3 + 2 * n_short || plain_total == 0) {
+    return plain;
+  }
+  WideTiling mixed;
+  mixed.full_x = (unsigned)((units - 2 * n_short) / 3);
+  mixed.short_x = n_short;
+  const size_t full_total = mixed.full_x * rows, total = full_total + n_short * rows;
+  mixed.grid = (unsigned)(total < resident ? total : resident);
+  // block i computes the tiles i, i + grid, ...: the longest one is among the first
+  // (one tile more) or holds the most full tiles
+  const double short_work = (double)kWideShortBX / kWideBX, change = 0.05;
+  mixed.rounds = 0.0;
+  for (size_t i = 0; i < mixed.grid; ++i) {
+    const size_t mine = (total - i + mixed.grid - 1) / mixed.grid;
+    const size_t full = i < full_total ? (full_total - i + mixed.grid - 1) / mixed.grid : 0;
+    const double work = (double)full + short_work * (double)(mine - full) + (full > 0 && mine > full ? change : 0.0);
+    mixed.rounds = work > mixed.rounds ? work : mixed.rounds;
+  }
+  return mixed.rounds < plain.rounds ? mixed : plain;
+}
+
 // The 192 x 256 block of gemm_mfma_wide.h (16-bit input; tiled layout, or IL: the
 // pipeline's interleaved rows): one persistent block per compute unit.
 template <int DT, int TOUT, bool IL = false>
 hipError_t launch_wide(const GemmParams &p, hipStream_t stream) {
-  const KernelArgs a = make_kernel_args(p, kWideBX, kWideBY);
-  const size_t total = (size_t)a.blocks_x * a.blocks_y * p.batch;
+  KernelArgs a = make_kernel_args(p, kWideBX, kWideBY);
+  const WideTiling tiling = wide_tiling(p);
+  a.blocks_x = tiling.full_x;
+  a.short_x = tiling.short_x;
+  const size_t total = (size_t)(a.blocks_x + a.short_x) * a.blocks_y * p.batch;
   if (total == 0) return hipSuccess;
   if (hipError_t e = check_grid(total)) return e;
-  const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
-  const unsigned grid = (unsigned)(total < resident ? total : resident);
+  const unsigned grid = tiling.grid;
   if (p.have_alpha) {
-    // (interleaved rows, alpha and a 16-bit C together need more registers than a
-    // lane has; wide_tiles_apply keeps that combination away)
-    if constexpr (IL && TOUT != kFloat32) {
-      return hipErrorInvalidValue;
-    } else {
-      auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL, true>;
-      static std::atomic<bool> lds_allowed[kMaxDevices];
-      if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
-      hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
-    }
+    auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL, true>;
+    static std::atomic<bool> lds_allowed[kMaxDevices];
+    if (hipError_t e = allow_lds(kernel, kWideLdsBytes, lds_allowed)) return e;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
   } else {
     auto kernel = complex_gemm_mfma_wide<DT, TOUT, IL, false>;
     static std::atomic<bool> lds_allowed[kMaxDevices];
@@ -2049,7 +2093,6 @@ inline bool wide_tiles_apply(const GemmParams &p) {
     return false;
   }
   if (p.input_interleaved) {
-    if (p.have_alpha && p.type_out != kFloat32) return false;   // (registers, see launch_wide)
     // rows of whole 128-byte pieces (32 complex values), at least two of them; a
     // lane's offset inside a copy of 8 rows is a 32-bit number
     const size_t row_bytes = (size_t)2 * p.k * bits_of(p.type_in) / 8;
@@ -2067,9 +2110,11 @@ inline bool wide_tiles_pay(const GemmParams &p) {
     const size_t tiles = (size_t)p.batch * cols * rows;
     return (double)p.batch * p.nx * p.ny / (double)(units * ceil_div(tiles, units) * bx * by);
   };
+  const double wide_useful =
+      (double)p.batch * p.nx * p.ny / ((double)units * wide_tiling(p).rounds * kWideBX * kWideBY);
   const double other = useful(256, 128) > useful(128, 128) / 1.15 ? useful(256, 128)
                                                                    : useful(128, 128) / 1.15;
-  return useful(kWideBX, kWideBY) * 1.075 > other;
+  return wide_useful * 1.075 > other;
 }
 
 template <int DT, int TOUT>

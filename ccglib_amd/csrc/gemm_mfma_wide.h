@@ -35,6 +35,10 @@
 //    keeps the order of complex_gemm_mfma_dtl (Xr Yr before Xi Yi, Xr Yi before
 //    Xi Yr), so both kernels produce the same bits.
 //
+//  * Where 192 does not divide the width of C, the last one or two tiles of a row
+//    of tiles can be short ones of 128 columns (see WideTile): 8 instead of 12 X
+//    tiles per K iteration, with a K loop of their own.
+//
 // Included by gemm_mfma.hip inside its namespaces, after the helpers it uses.
 #ifndef CCGLIB_AMD_GEMM_MFMA_WIDE_H_
 #define CCGLIB_AMD_GEMM_MFMA_WIDE_H_
@@ -44,6 +48,7 @@ constexpr int kWideXSlots = 3, kWideYSlots = 2;
 constexpr int kWideLdsBytes =
     (kWideXSlots * 2 * kWideBX + kWideYSlots * 2 * kWideBY) * kTileRowBytes;   // 136 KiB
 constexpr int kWideTX = kWideBX / 16;   // X tiles of a wave
+constexpr int kWideShortBX = 128;       // columns of a short tile: the first eight X tiles
 
 // The MFMA as an inline-asm statement with the register file of the accumulator
 // spelled out. The compiler puts the accumulators of all matrix instructions of a
@@ -116,21 +121,51 @@ __device__ __forceinline__ void take_accumulators(float4_t &a, float4_t &b, floa
   }
 }
 
-// tile_coord for a tile id that differs from lane to lane (plain divisions).
-__device__ __forceinline__ TileCoord tile_coord_by_lane(const KernelArgs &args, unsigned wg) {
+// The C tiles of a launch: args.blocks_x tiles of 192 columns per row of tiles,
+// followed - where 192 does not divide the width of C and the host found that it
+// pays - by args.short_x tiles of 128 columns (4096 = 20 x 192 + 2 x 128) instead of
+// one tile that hangs over the edge. All full tiles come first in the numbering,
+// in the order of tile_coord; the short ones follow, so that a block, which walks
+// the numbering with the stride of the grid, meets its full tiles before its short
+// ones. A tile is named by its batch, its first column and its row of tiles.
+struct WideTile {
+  unsigned b, x0, block_y;
+};
+// BY_LANE: the tile id differs from lane to lane (plain divisions).
+template <bool BY_LANE>
+__device__ __forceinline__ WideTile wide_tile(const KernelArgs &args, unsigned id) {
+  const unsigned full = args.blocks_x * args.blocks_y * args.batch;
+  WideTile w;
+  if (id >= full) {
+    // short tiles of one row of tiles are neighbours; rows of a batch follow each other
+    const unsigned r = xcd_remap(id - full, args.short_x * args.blocks_y * args.batch);
+    const unsigned row = r / args.short_x;
+    w.x0 = args.blocks_x * kWideBX + (r % args.short_x) * kWideShortBX;
+    w.block_y = row % args.blocks_y;
+    w.b = row / args.blocks_y;
+    if constexpr (!BY_LANE) {
+      w.b = (unsigned)__builtin_amdgcn_readfirstlane((int)w.b);
+      w.x0 = (unsigned)__builtin_amdgcn_readfirstlane((int)w.x0);
+      w.block_y = (unsigned)__builtin_amdgcn_readfirstlane((int)w.block_y);
+    }
+    return w;
+  }
+  if constexpr (!BY_LANE) {
+    const TileCoord tc = tile_coord(args, id);
+    return WideTile{tc.b, tc.block_x * kWideBX, tc.block_y};
+  }
   const unsigned per_batch = args.blocks_x * args.blocks_y;
-  const unsigned logical = xcd_remap(wg, per_batch * args.batch);
-  TileCoord tc;
-  tc.b = logical / per_batch;
+  const unsigned logical = xcd_remap(id, full);
+  w.b = logical / per_batch;
   const unsigned t = logical % per_batch;
   constexpr unsigned GROUP = 4;
   const unsigned group_size = GROUP * args.blocks_x;
   const unsigned g = t / group_size, in_group = t % group_size;
   const unsigned first_y = g * GROUP;
   const unsigned rows_in_group = (args.blocks_y - first_y) < GROUP ? (args.blocks_y - first_y) : GROUP;
-  tc.block_y = first_y + in_group % rows_in_group;
-  tc.block_x = in_group / rows_in_group;
-  return tc;
+  w.block_y = first_y + in_group % rows_in_group;
+  w.x0 = in_group / rows_in_group * kWideBX;
+  return w;
 }
 
 
@@ -150,6 +185,19 @@ __device__ __forceinline__ TileCoord tile_coord_by_lane(const KernelArgs &args, 
 // four), so the chunk swizzles of that layout carry over.
 // ALPHA: the result is multiplied by the complex alpha of the arguments on its way
 // out (both parts of an element sit in the same lane, in acc_re and acc_im).
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in this order.
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_each(std::integer_sequence<int, Is...>, F &&f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_each(std::make_integer_sequence<int, N>{}, f);
+}
+
+// (the lambdas of the kernel: left to its cost estimate, the compiler keeps the larger
+// ones as functions in some instantiations, and the accumulators then live in memory)
+#define CCGLIB_INLINE __attribute__((always_inline))
 template <int DT, int TOUT, bool IL, bool ALPHA>
 __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArgs args) {
   static_assert(DtypeTraits<DT>::kTilesPerMfma == 1 && DtypeTraits<DT>::kElemBytes == 2,
@@ -176,34 +224,39 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // kernel for rows of whole 128-byte pieces)
   const unsigned k_tiles = IL ? args.k_tiles / 2 : args.k_tiles;
   const unsigned row_stride = 2 * args.row_stride_bytes;   // IL: bytes from row to row
-  const unsigned total = args.blocks_x * args.blocks_y * args.batch;
+  const unsigned full_total = args.blocks_x * args.blocks_y * args.batch;
+  const unsigned total = full_total + args.short_x * args.blocks_y * args.batch;
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
 
   // ---- the C tiles of this block -------------------------------------------------
-  // Tile n of the block is C tile blockIdx.x + n gridDim.x. Lane n works out the
+  // Tile n of the block is C tile blockIdx.x + n gridDim.x; the short tiles are the
+  // last ones in the numbering, so a block meets its full tiles first. Lane n works out the
   // coordinates of tile n once (the first 64; a block with more takes the slow
   // way for the rest), and the wave fetches them with a lane read at every tile
   // change: with one wave per SIMD the divisions would otherwise stand in the
   // middle of the MFMA stream.
-  const unsigned my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  const unsigned first_tile = blockIdx.x, tile_stride = gridDim.x;
+  const unsigned my_tiles = (total - first_tile + tile_stride - 1) / tile_stride;
+  const unsigned my_full_tiles =
+      first_tile < full_total ? (full_total - first_tile + tile_stride - 1) / tile_stride : 0;
   unsigned table_b, table_x, table_y;
   {
-    unsigned vt = blockIdx.x + (unsigned)lane * gridDim.x;
-    vt = vt < total ? vt : blockIdx.x;
-    const TileCoord tc = tile_coord_by_lane(args, vt);
+    unsigned vt = first_tile + (unsigned)lane * tile_stride;
+    vt = vt < total ? vt : first_tile;
+    const WideTile tc = wide_tile<true>(args, vt);
     table_b = tc.b;
-    table_x = tc.block_x;
+    table_x = tc.x0;
     table_y = tc.block_y;
   }
   auto coords = [&](unsigned n) {   // past the last tile: the last one again (copied, never used)
     n = n < my_tiles ? n : my_tiles - 1;
-    TileCoord tc;
+    WideTile tc;
     if (n < 64) {
       tc.b = (unsigned)__builtin_amdgcn_readlane((int)table_b, (int)n);
-      tc.block_x = (unsigned)__builtin_amdgcn_readlane((int)table_x, (int)n);
+      tc.x0 = (unsigned)__builtin_amdgcn_readlane((int)table_x, (int)n);
       tc.block_y = (unsigned)__builtin_amdgcn_readlane((int)table_y, (int)n);
     } else {
-      tc = tile_coord(args, blockIdx.x + n * gridDim.x);
+      tc = wide_tile<false>(args, first_tile + n * tile_stride);
     }
     return tc;
   };
@@ -250,13 +303,13 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // wave-uniform: K tile 0 of the operand tile that holds row block i of the wave's
   // six of X; K tile 0 of the wave's rows of Y (re plane)
   const char *x_src[6], *y_src = nullptr;
-  auto point_x = [&](unsigned n) {
-    const TileCoord tc = coords(n);
+  auto point_x = [&](unsigned n) CCGLIB_INLINE {
+    const WideTile tc = coords(n);
     if constexpr (IL) {
       const char *op = args.x + (size_t)tc.b * args.x_batch_bytes;
 #pragma unroll
       for (int i = 0; i < 6; ++i) {
-        unsigned row0 = tc.block_x * BX + (6 * wave + i) * 8;
+        unsigned row0 = tc.x0 + (6 * wave + i) * 8;
         row0 = row0 < args.nx ? row0 : args.nx - 8;   // rows past the end: never stored
         x_src[i] = op + (size_t)row0 * row_stride;
       }
@@ -265,15 +318,15 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     const char *op = args.x + (size_t)tc.b * args.x_batch_bytes + x_plane * kTilePlaneBytes;
 #pragma unroll
     for (int i = 0; i < 6; ++i) {
-      const unsigned row0 = tc.block_x * BX + (x_rb0 + i) * 16;
+      const unsigned row0 = tc.x0 + (x_rb0 + i) * 16;
       unsigned tile = row0 / kTileRows;
       tile = tile < args.x_tiles ? tile : args.x_tiles - 1;   // rows past the end: never stored
       x_src[i] = op + (size_t)tile * args.k_tile_stride * kTileBytes +
                  (row0 % kTileRows) * kTileRowBytes;
     }
   };
-  auto point_y = [&](unsigned n) {
-    const TileCoord tc = coords(n);
+  auto point_y = [&](unsigned n) CCGLIB_INLINE {
+    const WideTile tc = coords(n);
     const unsigned row0 = tc.block_y * BY + wave * 64;
     if constexpr (IL) {
       y_src = args.y + (size_t)tc.b * args.y_batch_bytes +
@@ -289,7 +342,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // 8 - 13 its row blocks of X. One at a time and well apart: every vector memory
   // instruction occupies the compute unit's address unit for 16 cycles, and a wave
   // that issues the next one earlier waits - with its matrix instructions behind it.
-  auto issue = [&](int c, unsigned x_slot, unsigned y_slot) {
+  auto issue = [&](int c, unsigned x_slot, unsigned y_slot) CCGLIB_INLINE {
     if constexpr (IL) {
       // 0 - 7: rows 8 c .. 8 c + 7 of the wave's 64 of Y; 8 - 13: its 8-row blocks of X
       if (c < 8) {
@@ -312,13 +365,13 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
                      x_lds + x_slot * X_BYTES + i * 1024);
     }
   };
-  auto advance_x = [&] {
+  auto advance_x = [&]() CCGLIB_INLINE {
     if (++xs.kt == k_tiles) {
       xs.kt = 0;
       point_x(++xs.n);
     }
   };
-  auto advance_y = [&] {
+  auto advance_y = [&]() CCGLIB_INLINE {
     if (++ys.kt == k_tiles) {
       ys.kt = 0;
       point_y(++ys.n);
@@ -367,17 +420,17 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // does not insert the wait states that such a read needs after a vector-ALU
   // write: the instruction then sees the old register contents. With it, every
   // derived value is written several matrix instructions before its first use.
-  auto swap_pairs = [](int v) {
+  auto swap_pairs = [](int v) CCGLIB_INLINE {
     int o = (int)__builtin_amdgcn_alignbit((unsigned)v, (unsigned)v, 16);
     asm volatile("" : "+v"(o));
     return o;
   };
-  auto flip_sign = [](int v, int mask) {
+  auto flip_sign = [](int v, int mask) CCGLIB_INLINE {
     int o = v ^ mask;
     asm volatile("" : "+v"(o));
     return o;
   };
-  auto flip = [&](const int4_t &v) {
+  auto flip = [&](const int4_t &v) CCGLIB_INLINE {
     int4_t o;
 #pragma unroll
     for (int w = 0; w < 4; ++w) o[w] = flip_sign(v[w], (int)DtypeTraits<DT>::kSignMask);
@@ -407,8 +460,6 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     xn[0] = flip(xi[0]);
   }
 
-  float4_t acc_re[4][TX], acc_im[4][TX];
-
   // ---- the C stores ----------------------------------------------------------------
   // A wave's 192 x 64 patch leaves in 96 store instructions of four 256-byte row
   // segments (see store_piece), none of them after the K loop: they are issued one
@@ -432,24 +483,40 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   const unsigned lane_store_off =
       (unsigned)((((lane >> 4) * 4) * (size_t)args.nx + (lane & 15) * 4) * sizeof(Tout));
   const size_t plane_bytes = (size_t)args.nx * args.ny * sizeof(Tout);
-  auto aim_stores = [&](unsigned n) {
-    const TileCoord tc = coords(n);
-    const unsigned x_block = tc.block_x * BX, y_wave = tc.block_y * BY + wave * 64;
+  auto aim_stores = [&](unsigned n, bool short_tile) CCGLIB_INLINE {
+    const WideTile tc = coords(n);
+    const unsigned x_block = tc.x0, y_wave = tc.block_y * BY + wave * 64;
     target.base = args.c + ((size_t)tc.b * 2 * args.nx * args.ny + (size_t)y_wave * args.nx + x_block) *
                                sizeof(Tout);
     const bool y_in = y_wave < args.ny;
     target.inside[0] = y_in;
     target.inside[1] = y_in && x_block + 64 < args.nx;
-    target.inside[2] = y_in && x_block + 128 < args.nx;
-    target.all = target.inside[2];
+    target.inside[2] = y_in && !short_tile && x_block + 128 < args.nx;
+    target.all = short_tile ? target.inside[1] : target.inside[2];
   };
+  // ---- the body: full tiles or short ones --------------------------------------------
+  // A block computes its full tiles, then its short ones, and each kind has its own
+  // copy of what follows, with its own accumulators; the copies of the operands
+  // run on from one to the other. All 256 AccVGPRs and 128 VGPRs are taken: where
+  // two chains of updates of the same accumulators met (one loop over tiles of both
+  // kinds, or short tiles that take over the stores of a full one) the compiler
+  // would have to fit the registers of one into the gaps of the other - it copies
+  // accumulators around instead, right behind matrix instructions whose wait states
+  // it does not know.
+  using Yes = std::true_type;
+  using No = std::false_type;
+  auto body = [&](auto narrow, unsigned n_begin, unsigned n_end) CCGLIB_INLINE {
+  constexpr bool SHORT = decltype(narrow)::value;
+  constexpr int TXK = SHORT ? kWideShortBX / 16 : TX;   // X tiles of a C tile
+  float4_t acc_re[4][TXK], acc_im[4][TXK];
+
   // Store s (0 .. 31) of group g: tile row j = s / 8, plane (s / 4) % 2, register e =
   // s % 4 of the group's four tiles, which are four consecutive x of row 16 j + 4
   // (lane / 16) + e. The empty asm statement takes the accumulators where they are,
   // here and now: without it the compiler may read them right behind the matrix
   // instruction that wrote them, whose wait states it does not know.
-  auto store_piece = [&](int g, int s) {
-    if (!target.inside[g]) return;
+  auto store_piece = [&](int g, int s) CCGLIB_INLINE {
+    if (!target.inside[g] || (SHORT && g >= 2)) return;
     const int j = s >> 3, plane = (s >> 2) & 1, e = s & 3;
     float v[4];
     if constexpr (ALPHA) {
@@ -459,7 +526,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
       if (g < 2) {
         take_accumulators<true>(acc_re[j][4 * g], acc_re[j][4 * g + 1], acc_re[j][4 * g + 2], acc_re[j][4 * g + 3]);
         take_accumulators<true>(acc_im[j][4 * g], acc_im[j][4 * g + 1], acc_im[j][4 * g + 2], acc_im[j][4 * g + 3]);
-      } else {
+      } else if constexpr (!SHORT) {
         take_accumulators<false>(acc_re[j][4 * g], acc_re[j][4 * g + 1], acc_re[j][4 * g + 2], acc_re[j][4 * g + 3]);
         take_accumulators<false>(acc_im[j][4 * g], acc_im[j][4 * g + 1], acc_im[j][4 * g + 2], acc_im[j][4 * g + 3]);
       }
@@ -470,16 +537,23 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         v[i] = plane == 0 ? alpha_times_re(ar, ai, re, im) : alpha_times_im(ar, ai, re, im);
       }
     } else {
-      float4_t(&acc)[4][TX] = plane == 0 ? acc_re : acc_im;
+      float4_t(&acc)[4][TXK] = plane == 0 ? acc_re : acc_im;
       if (g < 2) {
         take_accumulators<true>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
-      } else {
+      } else if constexpr (!SHORT) {
         take_accumulators<false>(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
       }
       v[0] = acc[j][4 * g][e];
       v[1] = acc[j][4 * g + 1][e];
       v[2] = acc[j][4 * g + 2][e];
       v[3] = acc[j][4 * g + 3][e];
+    }
+    if constexpr (!ALPHA) {
+      // The four values are gathered in ordinary registers. Left to itself the
+      // compiler gathers them in a tuple of AccVGPRs, and where every AccVGPR holds
+      // an accumulator it moves four of those out of the way and back - reading
+      // them right behind matrix instructions whose wait states it does not know.
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
     }
     char *p = target.base + plane * plane_bytes +
               ((size_t)(j * 16 + e) * args.nx + g * 64) * sizeof(Tout) + lane_store_off;
@@ -494,16 +568,24 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
       __builtin_nontemporal_store(__builtin_bit_cast(ushort4_t, t4), reinterpret_cast<ushort4_t *>(p));
     }
   };
-  constexpr int kStoresPerIteration = 48;
+  constexpr int kStoresPerIteration = 4 * TXK;   // half of a tile's stores
 
   // One K iteration. `first`: the first one of a C tile (sums start from zero);
   // written out on its own, so that the accumulators have one definition there and
-  // one chain of updates in the loop over the middle ones. `carry`: a first
-  // iteration that issues the remaining stores of the previous C tile. `last`:
-  // the last one of a C tile, which issues the first half of its stores.
-  auto iteration = [&](auto first, auto carry, auto last) {
-    constexpr bool FIRST = decltype(first)::value, CARRY = decltype(carry)::value,
-                   LAST = decltype(last)::value;
+  // one chain of updates in the loop over the middle ones. It also issues the
+  // remaining stores of the previous C tile; for the block's first tile the target
+  // is still the empty one and every store is skipped (a second variant without
+  // the stores would meet this one where the loop begins - two chains of
+  // definitions, see above). `last`: the last one of a C tile, which issues the
+  // first half of its stores.
+  // A short tile: the first eight X tiles only, the same 14 copies (the X rows past
+  // the tile are fetched and not used) one every 8 instead of 12 matrix
+  // instructions, the boundary inside X tile 7; its stores are those of group 0 in
+  // the last iteration and those of group 1 in the next first one.
+  auto iteration = [&](auto first, auto last) CCGLIB_INLINE {
+    constexpr bool FIRST = decltype(first)::value, CARRY = FIRST, LAST = decltype(last)::value;
+    constexpr int TXI = TXK;
+    constexpr int kCopyEvery = SHORT ? 8 : 12;
     // the bookkeeping (which branches at a C tile change) of the copies issued
     // inside this iteration: K tile + 2 of both operands
     advance_y();
@@ -514,9 +596,9 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     const unsigned ya_next = yo + (y_slot ^ 1) * Y_BYTES;
 #define CCGLIB_PIN __builtin_amdgcn_sched_barrier(0)
     // what else is issued behind MFMA p of tile t
-    auto behind = [&](int t, int p) {
+    auto behind = [&](int t, int p) CCGLIB_INLINE {
       const int s = t & 1;
-      if (t + 1 < TX) {
+      if (t + 1 < TXI) {
         // the next tile's X fragments into the other register set
         if (p == 0) {
           const unsigned a = xo[(t + 1) & 3] + xa + ((t + 1) >> 2) * GROUP;
@@ -537,7 +619,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         // both variants of the next tile's fragments (the next iteration's first
         // tile behind the last one), two instructions behind each of eight MFMAs;
         // the exchange reads the raw value, so it comes before the sign flip
-        const int ns = t + 1 < TX ? (s ^ 1) : 0, w = 2 * (p & 1);
+        const int ns = t + 1 < TXI ? (s ^ 1) : 0, w = 2 * (p & 1);
         CCGLIB_PIN;
         if (p < 10) {
           xn[ns][w] = swap_pairs(xr[ns][w]);
@@ -565,40 +647,53 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         }
         if (CARRY && (idx & 1) && idx < 1 + 2 * kStoresPerIteration) {
           const int s = (idx - 1) / 2;
-          store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+          if (SHORT) {
+            store_piece(1, s);
+          } else {
+            store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+          }
           CCGLIB_PIN;
         }
       }
       {
-        // The copy of K tile + 2, one instruction every 12 MFMAs from tile 1 on: the
+        // The copy of K tile + 2, one instruction every 12 (8) MFMAs from tile 1 on: the
         // Y slot whose fragments this iteration holds in registers, and the X slot
         // that the barrier of the previous iteration's last tile released.
         const int m = 16 * t + p - 16;
-        if (m >= 0 && m % 12 == 6 && m / 12 < kCopies) {
-          issue(m / 12, x_refill, y_slot);
+        if (m >= 0 && m % kCopyEvery == 6 && m / kCopyEvery < kCopies) {
+          issue(m / kCopyEvery, x_refill, y_slot);
           CCGLIB_PIN;
         }
       }
-      if (t == TX - 1) {
+      if (t == TXI - 1) {
         // The iteration boundary. MFMA 4 of the last tile has waited for the
         // wave's last fragment read from this X slot (IL: MFMA 0 has, whose operand
         // was computed from it; the boundary is at MFMA 1 there, so that the two
         // variants of the next fragments can be made behind MFMAs 8 - 15 as in
-        // every other tile - one copy of this iteration is then still to come).
+        // every other tile). Copy c goes out behind MFMA 22 + 12 c (22 + 8 c) of the
+        // iteration: 14 of them before the boundary, or 13 (IL), or 12 (short tile) -
+        // the rest of this iteration's copies is then still to come.
         constexpr int kBoundary = IL ? 1 : 4;
-        constexpr int kCopiesBefore = IL ? kCopies - 1 : kCopies;
-        static_assert(22 + 12 * (kCopiesBefore - 1) <= 16 * (TX - 1) + kBoundary &&
-                          (kCopiesBefore == kCopies || 22 + 12 * kCopiesBefore > 16 * (TX - 1) + kBoundary),
-                      "copies issued before the boundary");
+        constexpr int kAllBefore = (16 * (TXI - 1) + kBoundary - 22) / kCopyEvery + 1;
+        constexpr int kCopiesBefore = kAllBefore < kCopies ? kAllBefore : kCopies;
+        static_assert(kCopiesBefore == (SHORT ? 12 : IL ? 13 : 14), "copies issued before the boundary");
+        static_assert(22 + kCopyEvery * (kCopies - 1) < 16 * TXI, "every copy inside the iteration");
+        // stores of this iteration issued before the boundary: behind the odd MFMAs
+        // from 65 (last iteration) or 1 (first) on, up to the boundary's own
+        constexpr int kIdxBoundary = 16 * (TXI - 1) + kBoundary;
+        constexpr int kLastOdd = kIdxBoundary % 2 ? kIdxBoundary : kIdxBoundary - 1;
+        constexpr int kSoFar = (kLastOdd - (LAST ? 65 : 1)) / 2 + 1;
+        constexpr int kStoresBefore = kSoFar < kStoresPerIteration ? kSoFar : kStoresPerIteration;
+        static_assert(kStoresBefore == (!SHORT || !LAST ? kStoresPerIteration : IL ? 25 : 26), "stores before the boundary");
         if (p == kBoundary) {
           // This wave's copies of the next K tile are complete when nothing older
           // than the requests of this iteration is outstanding - which are its
           // copies and, in a first or last iteration of a tile that lies entirely
-          // inside C, its 48 stores (the counter retires loads in order and does
+          // inside C, its stores so far (the counter retires loads in order and does
           // not tell them from stores; where stores may have been skipped, the
           // smaller number is the safe one and waits for more than it has to).
           if ((CARRY || LAST) && target.all) {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesBefore + kStoresPerIteration) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesBefore + kStoresBefore) : "memory");
           } else {
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kCopiesBefore) : "memory");
           }
@@ -627,8 +722,11 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         }
       }
     };
-#pragma unroll
-    for (int t = 0; t < TX; ++t) {
+    // (one copy of the loop body per X tile, made by the template and not left to the
+    // unroller: past a size limit that one leaves the loop as it is, and the
+    // accumulators, then indexed at run time, would live in memory)
+    static_for<TXI>([&](auto x_tile) CCGLIB_INLINE {
+      constexpr int t = decltype(x_tile)::value;
       const int s = t & 1;
       // exchanged roles: Y supplies the instruction's "A" rows, X its "B" columns
 #define CCGLIB_MM(ACC, Y, X, Z, P)                                                     \
@@ -656,7 +754,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
         CCGLIB_MM(acc_re[3][t], yi[3], xi[s], false, 13)
         CCGLIB_MM(acc_im[2][t], yi[2], xm[s], false, 14)
         CCGLIB_MM(acc_im[3][t], yi[3], xm[s], false, 15)
-        continue;
+        return;
       }
       CCGLIB_MM(acc_re[0][t], yr[0], xr[s], FIRST, 0)
       CCGLIB_MM(acc_re[1][t], yr[1], xr[s], FIRST, 1)
@@ -675,34 +773,39 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
       CCGLIB_MM(acc_re[2][t], yi[2], xn[s], false, 14)
       CCGLIB_MM(acc_re[3][t], yi[3], xn[s], false, 15)
 #undef CCGLIB_MM
-    }
+    });
 #undef CCGLIB_PIN
     x_slot = x_next;
     y_slot ^= 1;
   };
 
   // (k_tiles >= 2: the host does not launch this kernel for a K of one tile)
-  using Yes = std::true_type;
-  using No = std::false_type;
-  for (unsigned n = 0; n < my_tiles; ++n) {
-    if (n == 0) {
-      iteration(Yes{}, No{}, No{});
-    } else {
-      iteration(Yes{}, Yes{}, No{});
-    }
-    for (unsigned it = 2; it < k_tiles; ++it) iteration(No{}, No{}, No{});
-    aim_stores(n);
-    iteration(No{}, No{}, Yes{});
+  for (unsigned n = n_begin; n < n_end; ++n) {
+    iteration(Yes{}, No{});
+    for (unsigned it = 2; it < k_tiles; ++it) iteration(No{}, No{});
+    aim_stores(n, SHORT);
+    iteration(No{}, Yes{});
   }
   // the second half of the last tile's stores
   wait_for_mfma_results();
 #pragma unroll
   for (int s = 0; s < kStoresPerIteration; ++s) {
-    store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+    if (SHORT) {
+      store_piece(1, s);
+    } else {
+      store_piece(s < 16 ? 1 : 2, s < 16 ? 16 + s : s - 16);
+    }
     __builtin_amdgcn_sched_barrier(0);
   }
+  // (the next body's first iteration must not take these stores for its own)
+  target = StoreTarget{nullptr, {false, false, false}, false};
+  };   // body
+  if (my_full_tiles > 0) body(No{}, 0, my_full_tiles);
+  if (my_full_tiles < my_tiles) body(Yes{}, my_full_tiles, my_tiles);
   // nothing may still be writing into LDS when the block gives it back
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
+
+#undef CCGLIB_INLINE
 
 #endif  // CCGLIB_AMD_GEMM_MFMA_WIDE_H_

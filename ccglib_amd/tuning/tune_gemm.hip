@@ -79,6 +79,15 @@ static hipError_t launch_popcount(const GemmParams &p, hipStream_t stream) {
 // counts) per 32 complex products of 8 "operations" each
 constexpr double kPopcountRoof = 256 * 64 * 2.4e9 * 32 / 1e12;   // 1258 TOP/s
 
+// the 192 x 256 kernel with tiles of 192 columns only (the last one hanging over the edge)
+template <int DT, int TOUT, bool IL>
+hipError_t launch_wide_full_tiles(const GemmParams &p, hipStream_t stream) {
+  g_wide_short_tiles = false;
+  const hipError_t e = launch_wide<DT, TOUT, IL>(p, stream);
+  g_wide_short_tiles = true;
+  return e;
+}
+
 // name: type, [operand layout,] block BX x BY, wave WX x WY, ring slots, MFMA rows
 static const std::vector<Config> kConfigs = {
 #ifndef TUNE_GEMM_SMALL
@@ -88,6 +97,7 @@ static const std::vector<Config> kConfigs = {
     {"f16 128x256 w64x64 s3 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true>, kFloat16, kFloat32},
     {"f16 128x256 w64x64 y3 x4 m16 xt", launch_dtl<kFloat16, kFloat32, 128, 256, 64, 64, 3, 2, kLoadTiled, 16, true, 4>, kFloat16, kFloat32},
     {"f16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32, false>, kFloat16, kFloat32},
+    {"f16 192x256 ... 1wave, full tiles only", launch_wide_full_tiles<kFloat16, kFloat32, false>, kFloat16, kFloat32},
     {"bf16 256x128 w64x64 s3 m16 xt", launch_dtl<kBfloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadTiled, 16, true>, kBfloat16, kFloat32},
     {"bf16 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32, false>, kBfloat16, kFloat32},
 #ifndef TUNE_GEMM_SMALL
@@ -113,6 +123,7 @@ static const std::vector<Config> kConfigs = {
 #endif
     {"f16 interleaved 256x128 w64x64 s3 m16", launch_dtl<kFloat16, kFloat32, 256, 128, 64, 64, 3, 2, kLoadInterleavedVec, 16>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"f16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kFloat16, kFloat32, true>, kFloat16, kFloat32, kLoadInterleavedVec},
+    {"f16 interleaved 192x256 ... 1wave, full tiles only", launch_wide_full_tiles<kFloat16, kFloat32, true>, kFloat16, kFloat32, kLoadInterleavedVec},
     {"bf16 interleaved 192x256 w192x64 x3 y2 m16 xt 1wave", launch_wide<kBfloat16, kFloat32, true>, kBfloat16, kFloat32, kLoadInterleavedVec},
 #ifndef TUNE_GEMM_SMALL
     {"fp8 planar 256x128 w64x64 s3 m32", launch_dtl<kFloat8e4m3, kFloat32, 256, 128, 64, 64, 3, 2, kLoadPlanarVec, 32>, kFloat8e4m3, kFloat32, kLoadPlanarVec},
@@ -482,9 +493,7 @@ int main(int argc, char **argv) {
     p.beta_im = 0;
     p.have_alpha = 0;
     p.have_beta = 0;
-    if (c.launch == launch_wide<kFloat16, kFloat32, false> || c.launch == launch_wide<kBfloat16, kFloat32, false> ||
-        c.launch == launch_wide<kFloat16, kFloat32, true> ||
-        c.launch == launch_wide<kBfloat16, kFloat32, true>) {
+    if (std::strstr(c.name, "192x256") != nullptr) {
       if (!wide_tiles_apply(p)) {
         std::printf("%-44s (not applicable to this shape)\n", c.name);
         continue;

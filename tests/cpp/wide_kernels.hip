@@ -16,6 +16,7 @@ CCGLIB_WIDE(kFloat16, kFloat32, true, true)
 CCGLIB_WIDE(kFloat16, kFloat16, false, false)
 CCGLIB_WIDE(kFloat16, kFloat16, false, true)
 CCGLIB_WIDE(kFloat16, kFloat16, true, false)
+CCGLIB_WIDE(kFloat16, kFloat16, true, true)
 CCGLIB_WIDE(kBfloat16, kFloat32, false, false)
 CCGLIB_WIDE(kBfloat16, kFloat32, false, true)
 CCGLIB_WIDE(kBfloat16, kFloat32, true, false)
@@ -23,6 +24,7 @@ CCGLIB_WIDE(kBfloat16, kFloat32, true, true)
 CCGLIB_WIDE(kBfloat16, kBfloat16, false, false)
 CCGLIB_WIDE(kBfloat16, kBfloat16, false, true)
 CCGLIB_WIDE(kBfloat16, kBfloat16, true, false)
+CCGLIB_WIDE(kBfloat16, kBfloat16, true, true)
 #undef CCGLIB_WIDE
 }  // namespace
 }  // namespace ccglib_amd

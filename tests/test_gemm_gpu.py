@@ -527,8 +527,9 @@ def test_wide_block_tile(tin, tout, c_order):
     """GEMM_BLOCK_TILE = 3: the 192 x 256 block (16-bit tiled input, planar C without
     beta, M and N multiples of 64, K of more than one tile) against the
     oracle: tiles that lie inside C and tiles of which only one or two 64-column
-    groups or some of the four 64-row pieces do, two to many K tiles, more C tiles
-    than compute units, and a K with a partial last tile."""
+    groups or some of the four 64-row pieces do, widths that end in one or two short
+    tiles of 128 columns, two to many K tiles, more C tiles than compute units, and a K
+    with a partial last tile."""
     with cc.option(cc.Option.gemm_block_tile, 3):
         float_case(2, 256, 192, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=1)
         float_case(3, 320, 448, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=2)
@@ -538,6 +539,12 @@ def test_wide_block_tile(tin, tout, c_order):
         # with a complex alpha (applied to the accumulators on their way out)
         float_case(3, 320, 448, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=1.5 - 0.5j, seed=6)
         float_case(2, 256, 192, 2048, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=-0.25 + 2j, seed=7)
+        # 448 = 192 + 2 x 128 columns: 90 full tiles and 180 short ones, more tiles than compute
+        # units (blocks with a full tile and then a short one, blocks with one short tile); then
+        # 150 full and 300 short tiles (blocks with two short tiles)
+        n, m = (448, 256) if c_order == ROW else (256, 448)
+        float_case(90, m, n, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=8)
+        float_case(150, m, n, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=0.5 + 0.5j, seed=9)
 
 
 def test_wide_block_tile_falls_back():

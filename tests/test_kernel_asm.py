@@ -10,10 +10,14 @@ needed) and checks what the source can only arrange for:
 * no vector-ALU instruction writes a register that a matrix instruction reads as its A or B
   operand within the two instructions before it (an operand derived from a fragment has to be
   computed several matrix instructions ahead; the hardware needs two wait states);
-* the scalar base address of a copy is not written by v_readlane / v_readfirstlane within the
-  three instructions before the copy's asm statement (a vector memory instruction may read a
-  scalar register five wait states after a vector-ALU instruction wrote it; the statement's
-  own s_mov and s_nop are two of them).
+* the scalar base address of a copy is written by a scalar move inside the copy's own asm
+  statement (a vector memory instruction may read a scalar register only five wait states
+  after a vector-ALU instruction - a v_readlane that reads a spilled scalar back - wrote it;
+  after the scalar ALU it may read it at once);
+* the compiler never writes an AccVGPR itself (v_accvgpr_write / v_accvgpr_mov: it would be
+  moving an accumulator out of the way or back, around matrix instructions whose wait states
+  it does not know), and reads one (for a C store) no sooner than four matrix instructions
+  after the last one that wrote it.
 """
 import os
 import re
@@ -48,7 +52,7 @@ def kernels():
             name = None
         elif name and s and not s.startswith((";", ".")) and not s.endswith(":"):
             found[name].append(s.split(";")[0].strip())
-    assert len(found) == 14
+    assert len(found) == 16
     return found, scratch
 
 
@@ -88,10 +92,10 @@ def test_matrix_operands_are_not_written_right_before_their_use(kernels):
                                                                    "v_readfirstlane")):
                     written = _registers(_operands(prev)[0], "va")
                     assert not (written & sources), (name, prev, ins)
-        assert n_mfma == 4 * 192     # the four variants of a K iteration
+        assert n_mfma == 3 * 192 + 3 * 128     # the three variants of a K iteration, full and short tiles
 
 
-def test_copy_base_is_not_fresh_out_of_a_vector_register(kernels):
+def test_copy_base_goes_through_a_scalar_move(kernels):
     found, _ = kernels
     for name, code in found.items():
         copies = 0
@@ -102,8 +106,26 @@ def test_copy_base_is_not_fresh_out_of_a_vector_register(kernels):
             base = _registers(_operands(ins)[1], "s")
             assert base, ins                      # a scalar register pair, not a vector one
             assert code[i - 2].startswith("s_mov_b32 m0") and code[i - 1].startswith("s_nop")
-            for back in (3, 4, 5):                # the three instructions before the statement
-                prev = code[i - back]
-                if prev.startswith(("v_readlane_b32", "v_readfirstlane_b32")):
-                    assert not (_registers(_operands(prev)[0], "s") & base), (name, prev, ins)
-        assert copies >= 2 * 14 + 4 * 14          # prologue and the four iteration variants
+            # written by the scalar ALU inside the same asm statement
+            assert code[i - 3].startswith("s_mov_b64"), (name, code[i - 3])
+            assert _registers(_operands(code[i - 3])[0], "s") == base, (name, code[i - 3], ins)
+        assert copies >= 2 * 14 + 6 * 14          # prologue and the six iteration variants
+
+
+def test_accumulators_stay_where_they_are(kernels):
+    found, _ = kernels
+    for name, code in found.items():
+        reads = 0
+        for i, ins in enumerate(code):
+            assert not ins.startswith(("v_accvgpr_write", "v_accvgpr_mov")), (name, ins)
+            if not ins.startswith("v_accvgpr_read"):
+                continue
+            reads += 1
+            source = _registers(_operands(ins)[1], "a")
+            seen, k = 0, i - 1
+            while seen < 4 and k >= 0 and not code[k].startswith("s_nop 15"):   # (the explicit wait)
+                if code[k].startswith("v_mfma"):
+                    seen += 1
+                    assert not (_registers(_operands(code[k])[0], "a") & source), (name, code[k], ins)
+                k -= 1
+        assert reads > 0

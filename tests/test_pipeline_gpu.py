@@ -478,7 +478,9 @@ def test_pipeline_interleaved_rows_wide_block(tin, tout, c_order):
     64-row pieces are, two to many K pieces, more C tiles than compute units."""
     for seed, (B, M, N, K, alpha) in enumerate([(2, 256, 192, 64, 1), (3, 320, 448, 96, 1),
                                                 (2, 512, 832, 992, 1), (40, 256, 576, 64, 1),
-                                                (1, 64, 64, 128, 1), (3, 320, 448, 96, 0.5 - 1.5j)]):
+                                                (1, 64, 64, 128, 1), (3, 320, 448, 96, 0.5 - 1.5j),
+                                                (90, 256, 448, 96, 1), (90, 448, 256, 64, 1),
+                                                (150, 256, 448, 64, 0.25 + 1j)]):
         rng = np.random.default_rng(40 + seed)
         qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), tin)
         qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), tin)
