@@ -229,8 +229,9 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
 
   // ---- the C tiles of this block -------------------------------------------------
-  // Tile n of the block is C tile blockIdx.x + n gridDim.x; the short tiles are the
-  // last ones in the numbering, so a block meets its full tiles first. Lane n works out the
+  // The block's C tiles are blockIdx.x + k gridDim.x; the short tiles are the last
+  // ones in the numbering, so these are full tiles up to some k and short ones from
+  // there. Lane n works out the
   // coordinates of tile n once (the first 64; a block with more takes the slow
   // way for the rest), and the wave fetches them with a lane read at every tile
   // change: with one wave per SIMD the divisions would otherwise stand in the
@@ -239,9 +240,20 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   const unsigned my_tiles = (total - first_tile + tile_stride - 1) / tile_stride;
   const unsigned my_full_tiles =
       first_tile < full_total ? (full_total - first_tile + tile_stride - 1) / tile_stride : 0;
+  // The order in which the block takes them: its short tiles before its full ones
+  // or after them, in turn for every four blocks of an XCD (the short tiles of one
+  // row of tiles and of a batch's neighbouring rows, which share operands). A short
+  // tile moves as many operand bytes as a full one for two thirds of the products:
+  // all of them at once, behind the full tiles, would wait for memory.
+  const unsigned short_begin = ((blockIdx.x / kNumXcd / 4) & 1) ? 0 : my_full_tiles;
+  const unsigned short_end = short_begin + (my_tiles - my_full_tiles);
+  auto tile_id = [&](unsigned n) {
+    const unsigned k = n < short_begin ? n : n < short_end ? my_full_tiles + (n - short_begin) : n - (short_end - short_begin);
+    return first_tile + k * tile_stride;
+  };
   unsigned table_b, table_x, table_y;
   {
-    unsigned vt = first_tile + (unsigned)lane * tile_stride;
+    unsigned vt = tile_id((unsigned)lane);
     vt = vt < total ? vt : first_tile;
     const WideTile tc = wide_tile<true>(args, vt);
     table_b = tc.b;
@@ -256,7 +268,7 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
       tc.x0 = (unsigned)__builtin_amdgcn_readlane((int)table_x, (int)n);
       tc.block_y = (unsigned)__builtin_amdgcn_readlane((int)table_y, (int)n);
     } else {
-      tc = wide_tile<false>(args, first_tile + n * tile_stride);
+      tc = wide_tile<false>(args, tile_id(n));
     }
     return tc;
   };
@@ -800,8 +812,13 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
   // (the next body's first iteration must not take these stores for its own)
   target = StoreTarget{nullptr, {false, false, false}, false};
   };   // body
-  if (my_full_tiles > 0) body(No{}, 0, my_full_tiles);
-  if (my_full_tiles < my_tiles) body(Yes{}, my_full_tiles, my_tiles);
+  // (written out: in a loop over the two kinds everything would be live everywhere)
+  if (short_begin == 0 && short_end > 0) body(Yes{}, 0, short_end);
+  if (my_full_tiles > 0) {
+    const unsigned first_full = short_begin == 0 ? short_end : 0;
+    body(No{}, first_full, first_full + my_full_tiles);
+  }
+  if (short_begin != 0 && short_end > short_begin) body(Yes{}, short_begin, short_end);
   // nothing may still be writing into LDS when the block gives it back
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }

@@ -92,7 +92,8 @@ def test_matrix_operands_are_not_written_right_before_their_use(kernels):
                                                                    "v_readfirstlane")):
                     written = _registers(_operands(prev)[0], "va")
                     assert not (written & sources), (name, prev, ins)
-        assert n_mfma == 3 * 192 + 3 * 128     # the three variants of a K iteration, full and short tiles
+        # the three variants of a K iteration, for full tiles and (two copies) for short ones
+        assert n_mfma == 3 * 192 + 6 * 128
 
 
 def test_copy_base_goes_through_a_scalar_move(kernels):
@@ -109,7 +110,7 @@ def test_copy_base_goes_through_a_scalar_move(kernels):
             # written by the scalar ALU inside the same asm statement
             assert code[i - 3].startswith("s_mov_b64"), (name, code[i - 3])
             assert _registers(_operands(code[i - 3])[0], "s") == base, (name, code[i - 3], ins)
-        assert copies >= 2 * 14 + 6 * 14          # prologue and the six iteration variants
+        assert copies >= 2 * 14 + 9 * 14          # prologue and the nine iteration variants
 
 
 def test_accumulators_stay_where_they_are(kernels):
