@@ -1996,11 +1996,14 @@ hipError_t launch_dtl(const GemmParams &p, hipStream_t stream) {
 
 // How the 192 x 256 kernel covers the width of C: tiles of 192 columns, the last of
 // which may hang over the edge, or - where 64 divides the width - full tiles
-// followed by one or two of 128 columns (4096 = 20 x 192 + 2 x 128), which take two
-// thirds of the matrix instructions. The short tiles are the last ones in the
-// kernel's numbering, and a block computes its full tiles before its short ones;
-// `rounds` is the work of the block that finishes last, in full tiles (B=64
-// 512x4096: 10 2/3 instead of 11), with a charge for the change of kind.
+// followed by short ones of 128 columns, which take two thirds of the matrix
+// instructions: as many as make the width come out even (4096 = 20 x 192 + 2 x 128),
+// or three more for two full ones less as long as that shortens the work of the
+// block that finishes last (8192 = 32 x 192 + 16 x 128: with 32 rows of tiles every
+// one of 256 blocks gets 4 full and 2 short tiles, 5 1/3 full tiles' worth, where
+// 42 x 192 + 128 would give 64 of them 6 full tiles). The short tiles are the last
+// ones in the kernel's numbering; `rounds` is that longest block's work in full
+// tiles, with a charge for the change of kind.
 struct WideTiling {
   unsigned full_x, short_x, grid;
   double rounds;
@@ -2010,33 +2013,33 @@ static bool g_wide_short_tiles = true;
 inline WideTiling wide_tiling(const GemmParams &p) {
   const size_t resident = (size_t)compute_units() / kNumXcd * kNumXcd;
   const size_t rows = ceil_div((size_t)p.ny, (size_t)kWideBY) * p.batch;
-  WideTiling plain;
-  plain.full_x = (unsigned)ceil_div((size_t)p.nx, (size_t)kWideBX);
-  plain.short_x = 0;
-  const size_t plain_total = plain.full_x * rows;
-  plain.grid = (unsigned)(plain_total < resident ? plain_total : resident);
-  plain.rounds = plain.grid ? (double)ceil_div(plain_total, (size_t)plain.grid) : 0.0;
+  WideTiling best;
+  best.full_x = (unsigned)ceil_div((size_t)p.nx, (size_t)kWideBX);
+  best.short_x = 0;
+  const size_t plain_total = best.full_x * rows;
+  best.grid = (unsigned)(plain_total < resident ? plain_total : resident);
+  best.rounds = best.grid ? (double)ceil_div(plain_total, (size_t)best.grid) : 0.0;
   const size_t units = p.nx / 64;
-  const unsigned n_short = units % 3 == 0 ? 0 : units % 3 == 2 ? 1 : 2;
-  if (!g_wide_short_tiles || p.nx % 64 != 0 || n_short == 0 || units < 3 + 2 * n_short || plain_total == 0) {
-    return plain;
-  }
-  WideTiling mixed;
-  mixed.full_x = (unsigned)((units - 2 * n_short) / 3);
-  mixed.short_x = n_short;
-  const size_t full_total = mixed.full_x * rows, total = full_total + n_short * rows;
-  mixed.grid = (unsigned)(total < resident ? total : resident);
-  // block i computes the tiles i, i + grid, ...: the longest one is among the first
-  // (one tile more) or holds the most full tiles
+  if (!g_wide_short_tiles || p.nx % 64 != 0 || plain_total == 0) return best;
   const double short_work = (double)kWideShortBX / kWideBX, change = 0.05;
-  mixed.rounds = 0.0;
-  for (size_t i = 0; i < mixed.grid; ++i) {
-    const size_t mine = (total - i + mixed.grid - 1) / mixed.grid;
-    const size_t full = i < full_total ? (full_total - i + mixed.grid - 1) / mixed.grid : 0;
-    const double work = (double)full + short_work * (double)(mine - full) + (full > 0 && mine > full ? change : 0.0);
-    mixed.rounds = work > mixed.rounds ? work : mixed.rounds;
+  for (size_t n_short = units % 3 == 0 ? 3 : units % 3 == 2 ? 1 : 2; 3 + 2 * n_short <= units; n_short += 3) {
+    WideTiling mixed;
+    mixed.full_x = (unsigned)((units - 2 * n_short) / 3);
+    mixed.short_x = (unsigned)n_short;
+    const size_t full_total = mixed.full_x * rows, total = full_total + n_short * rows;
+    mixed.grid = (unsigned)(total < resident ? total : resident);
+    // block i computes the tiles i, i + grid, ...
+    mixed.rounds = 0.0;
+    for (size_t i = 0; i < mixed.grid; ++i) {
+      const size_t mine = (total - i + mixed.grid - 1) / mixed.grid;
+      const size_t full = i < full_total ? (full_total - i + mixed.grid - 1) / mixed.grid : 0;
+      const double work =
+          (double)full + short_work * (double)(mine - full) + (full > 0 && mine > full ? change : 0.0);
+      mixed.rounds = work > mixed.rounds ? work : mixed.rounds;
+    }
+    if (mixed.rounds < best.rounds - 1e-9) best = mixed;
   }
-  return mixed.rounds < plain.rounds ? mixed : plain;
+  return best;
 }
 
 // The 192 x 256 block of gemm_mfma_wide.h (16-bit input; tiled layout, or IL: the
