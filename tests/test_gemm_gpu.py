@@ -545,6 +545,10 @@ def test_wide_block_tile(tin, tout, c_order):
         n, m = (448, 256) if c_order == ROW else (256, 448)
         float_case(90, m, n, 96, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=8)
         float_case(150, m, n, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, alpha=0.5 + 0.5j, seed=9)
+        # 4224 = 20 x 192 + 3 x 128 columns although 192 divides 4224: with 12 rows of tiles, 23
+        # tiles per row even out the work of the 256 blocks where 22 would not
+        n, m = (4224, 512) if c_order == ROW else (512, 4224)
+        float_case(6, m, n, 64, tin, tout, cc.Variant.opt, PLANAR, c_order, seed=10)
 
 
 def test_wide_block_tile_falls_back():
