@@ -137,12 +137,24 @@ def sample_core_clock(run, torch, load_s=1.2):
     tool = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
     if not os.path.exists(tool):
         return None
+    command = [tool, "--showclocks"]
+    try:
+        # rocm-smi is a Python script behind "#!/usr/bin/env python3": started with this
+        # interpreter directly, the child process is one program from start to end (under a
+        # profiler whose preloaded library touches the GPU in every process, the hop from
+        # env to python3 would replace a program that has initialised the GPU)
+        with open(tool, "rb") as f:
+            first = f.readline()
+        if first.startswith(b"#!") and b"python" in first:
+            command = [sys.executable, os.path.realpath(tool), "--showclocks"]
+    except OSError:
+        pass
     found = []
 
     def ask():
         time.sleep(load_s / 3)
         try:
-            out = subprocess.run([tool, "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+            out = subprocess.run(command, capture_output=True, text=True, timeout=20).stdout
             m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
             if m:
                 found.append(float(m.group(1)))

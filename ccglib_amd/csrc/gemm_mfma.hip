@@ -2087,9 +2087,10 @@ inline bool small_tiles_pay(const GemmParams &p, double penalty) {
 // Whether the 192 x 256 block of gemm_mfma_wide.h can compute this problem (what
 // its stores and its K loop assume), and whether it pays: per flop it measured
 // about 7 % faster than the 256 x 128 block once every compute unit is busy
-// (B=64 512x4096x576: 0.538 against 0.557 ms with 3 % of its tiles' columns
-// outside C), but its tiles are 1.5 times as large, so more of the last round of
-// tiles can stay empty (8192^3: 5.4 rounds of 192 x 256 tiles against 8 full ones).
+// (B=64 512x4096x576: 0.519 against 0.558 ms), but its tiles are 1.5 times as
+// large, so more of the last round of tiles can stay empty - which the short
+// tiles of wide_tiling even out where the width allows (8192^3: 5 1/3 tiles for
+// every block, 2.75 against 2.78 ms).
 inline bool wide_tiles_apply(const GemmParams &p) {
   if (p.c_interleaved || p.have_beta || (uintptr_t)p.c % 16 != 0 ||
       p.nx % 64 != 0 || p.ny % 64 != 0 || p.k_in_memory) {
