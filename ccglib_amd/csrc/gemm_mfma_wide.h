@@ -474,14 +474,16 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
 
   // ---- the C stores ----------------------------------------------------------------
   // A wave's 192 x 64 patch leaves in 96 store instructions of four 256-byte row
-  // segments (see store_piece), none of them after the K loop: they are issued one
-  // every other matrix instruction behind those of the tile's LAST K iteration and
-  // of the next tile's FIRST one, as the accumulators become final and before they
-  // are started again:
+  // segments (see store_piece), none of them after the K loop (but for a block's last
+  // tile of a kind): they are issued one every other matrix instruction behind those
+  // of the tile's LAST K iteration and of the next tile's FIRST one, as the
+  // accumulators become final and before they are started again:
   //   group 0 (X tiles 0 - 3, final behind tile 3 of the last iteration): last iteration;
   //   group 1 (tiles 4 - 7): half in the last iteration, half in the next first one
   //   (which starts these accumulators again with its tile 4);
   //   group 2 (tiles 8 - 11): the next first iteration, before its tile 8.
+  // (A short tile, 128 x 64 per wave: group 0 in its last iteration, group 1 in the
+  // next first one.)
   // The host only launches this kernel for planar C without beta, with
   // 16-byte aligned rows and nx, ny multiples of 64: a 64 x 64 piece of a tile is
   // either inside C or outside.
@@ -507,8 +509,8 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     target.all = short_tile ? target.inside[1] : target.inside[2];
   };
   // ---- the body: full tiles or short ones --------------------------------------------
-  // A block computes its full tiles, then its short ones, and each kind has its own
-  // copy of what follows, with its own accumulators; the copies of the operands
+  // A block computes its full tiles and its short ones one kind after the other, and
+  // each kind has its own copy of what follows, with its own accumulators; the copies of the operands
   // run on from one to the other. All 256 AccVGPRs and 128 VGPRs are taken: where
   // two chains of updates of the same accumulators met (one loop over tiles of both
   // kinds, or short tiles that take over the stores of a full one) the compiler
@@ -532,9 +534,8 @@ __global__ __launch_bounds__(256, 1) void complex_gemm_mfma_wide(const KernelArg
     const int j = s >> 3, plane = (s >> 2) & 1, e = s & 3;
     float v[4];
     if constexpr (ALPHA) {
-      // both parts of the four elements; the expressions of the other kernels'
-      // epilogues, so that the compiler contracts them alike and every block tile
-      // gives the same bits
+      // both parts of the four elements, through the helpers that every kernel's
+      // epilogue uses, so that every block tile gives the same bits
       if (g < 2) {
         take_accumulators<true>(acc_re[j][4 * g], acc_re[j][4 * g + 1], acc_re[j][4 * g + 2], acc_re[j][4 * g + 3]);
         take_accumulators<true>(acc_im[j][4 * g], acc_im[j][4 * g + 1], acc_im[j][4 * g + 2], acc_im[j][4 * g + 3]);
