@@ -581,6 +581,44 @@ def test_block_tile_choice_is_invisible(B, M, N, K, alpha):
         assert np.array_equal(results[0], r)
 
 
+def _same_bits_either_block_tile(B, M, N, K, seed, c_order=ROW, alpha=1):
+    rng = np.random.default_rng(seed)
+    qa = quantize(rng.uniform(-1, 1, (B, 2, M, K)).astype(np.float32), VT.float16).reshape(-1)
+    qb = quantize(rng.uniform(-1, 1, (B, 2, N, K)).astype(np.float32), VT.float16).reshape(-1)
+    results = []
+    for block_tile in (1, 3):
+        with cc.option(cc.Option.gemm_block_tile, block_tile):
+            results.append(run_gemm(qa, qb, B, M, N, K, VT.float16, VT.float32, cc.Variant.opt, PLANAR, c_order,
+                                    alpha))
+    assert np.array_equal(results[0], results[1]), (B, M, N, K, c_order)
+    return qa, qb, results[1]
+
+
+def test_wide_block_tilings_of_many_shapes():
+    """The 192 x 256 kernel covers the width of C with full tiles and short ones, and a block
+    takes its short tiles before or after its full ones: seeded random shapes (M, N multiples
+    of 64; from a few tiles to several per block, widths with none, one, two and more short
+    tiles per row of tiles) give the bits of the 256 x 128 kernel, which the other tests
+    compare with the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(14):
+        rows, cols = 64 * int(rng.integers(1, 13)), 64 * int(rng.integers(1, 40))
+        B = int(rng.integers(1, 1 + max(1, 2400 // ((rows + 255) // 256 * ((cols + 191) // 192)))))
+        K = int(rng.choice([64, 96, 160, 288]))
+        c_order = ROW if case % 3 else COL
+        M, N = (rows, cols) if c_order == ROW else (cols, rows)
+        _same_bits_either_block_tile(B, M, N, K, 100 + case, c_order, alpha=1 if case % 4 else 0.5 - 2j)
+
+
+def test_wide_block_more_than_64_tiles_with_short_ones():
+    """More than 64 tiles per block, short tiles among them (448 = 192 + 2 x 128 columns): the
+    coordinates past a block's table of 64, for tiles of both kinds."""
+    B, M, N, K = 6000, 64, 448, 64
+    qa, qb, got = _same_bits_either_block_tile(B, M, N, K, 13)
+    want = orc.gemm(qa[-3 * 2 * M * K:], qb[-3 * 2 * N * K:], M, N, K, ORC_TYPE[VT.float16], ORC_TYPE[VT.float32])
+    assert np.allclose(got[-3:], want.reshape(3, 2, M, N), rtol=1e-3, atol=1e-3)
+
+
 def test_wide_block_more_than_64_tiles_per_block():
     """A block of the 192 x 256 kernel looks the coordinates of its first 64 C tiles up in a
     table and works out the others one by one: 20000 one-tile batches are more than 64 tiles
