@@ -17,7 +17,8 @@ needed) and checks what the source can only arrange for:
 * the compiler never writes an AccVGPR itself (v_accvgpr_write / v_accvgpr_mov: it would be
   moving an accumulator out of the way or back, around matrix instructions whose wait states
   it does not know), and reads one (for a C store) no sooner than four matrix instructions
-  after the last one that wrote it.
+  after the last one that wrote it; the same distance holds for the accumulators that live in
+  ordinary registers and whatever reads them.
 """
 import os
 import re
@@ -130,3 +131,26 @@ def test_accumulators_stay_where_they_are(kernels):
                     assert not (_registers(_operands(code[k])[0], "a") & source), (name, code[k], ins)
                 k -= 1
         assert reads > 0
+
+
+def test_vgpr_accumulators_are_read_well_after_their_last_update(kernels):
+    found, _ = kernels
+    for name, code in found.items():
+        recent = []       # destination registers of the last four matrix instructions
+        checked = 0
+        for ins in code:
+            if ins.startswith("v_mfma"):
+                recent = (recent + [_registers(_operands(ins)[0], "v")])[-4:]
+                continue
+            if ins.startswith("s_nop 15"):      # (the explicit wait before a block's last stores)
+                recent = []
+                continue
+            live = set().union(*recent) if recent else set()
+            if not live or not ins.startswith(("v_", "global_", "ds_", "buffer_", "scratch_", "flat_")):
+                continue
+            ops = _operands(ins)
+            writes_first = not ins.startswith(("global_store", "ds_write", "ds_store", "buffer_store"))
+            for token in ops[1:] if writes_first else ops:
+                checked += 1
+                assert not (_registers(token, "v") & live), (name, ins)
+        assert checked > 0
